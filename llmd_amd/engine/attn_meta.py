@@ -14,6 +14,21 @@ import torch
 
 
 @dataclass
+class SeqMeta:
+    """Per-sequence description of a step for models whose layers keep per-sequence state or use
+    the per-row attention kernels (ops/seqmix.py): the step's tokens are the sequences' runs back
+    to back, decodes (one token each) first, then the prefill portions."""
+    num_seqs: int
+    seq_start: torch.Tensor          # [n + 1] int32: token bounds of each sequence's run
+    seq_slot: torch.Tensor           # [n] int32: state slot (engine/state_cache.py)
+    seq_init: torch.Tensor           # [n] int32: 1 = the slot holds this sequence's earlier state
+    row_seq: torch.Tensor            # [T] int32: token -> sequence (row of ``tables``)
+    row_len: torch.Tensor            # [T] int32: keys the token sees (= position + 1)
+    tables: torch.Tensor             # [n, W] int32 block tables
+    max_len: int = 0
+
+
+@dataclass
 class AttnMeta:
     num_tokens: int
     positions: torch.Tensor          # [T] int64
@@ -49,6 +64,8 @@ class AttnMeta:
     # hybrid KV cache (engine/hybrid_kv.py): the windowed layers' own slot mapping and
     # block tables (everything else shared), or None
     swa: Optional["AttnMeta"] = None
+    # per-sequence runs, state slots and per-row attention lengths (stateful / per-layer stacks)
+    seq: Optional[SeqMeta] = None
 
     @property
     def has_prefill(self) -> bool:

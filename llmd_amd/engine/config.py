@@ -67,6 +67,11 @@ class ModelConfig:
     # multimodal (llava-style: vision tower + LM; models/vision.py)
     vision_config: Optional[dict] = None
     image_token_id: int = 0
+    # per-layer stacks (models/mekusun.py): one entry per layer, {"type": mixer kind,
+    # "mixer": its sizes and constants, "mlp": feed-forward description or None}
+    layer_specs: Optional[list] = None
+    embedding_scale: float = 1.0
+    logit_softcap: float = 0.0
     name: str = "custom"
 
     def __post_init__(self):
@@ -106,6 +111,12 @@ class ModelConfig:
                 d = json.load(f)
         else:
             d = dict(path_or_dict)
+        if d.get("architecture") == "Mekusun":
+            shapes = {}
+            if isinstance(path_or_dict, (str, os.PathLike)):
+                st = os.path.join(os.path.dirname(p), "model.safetensors")
+                shapes = safetensors_shapes(st) if os.path.exists(st) else {}
+            return mekusun_config(d, shapes)
         names = {f.name for f in dataclasses.fields(cls)}
         kw = {k: v for k, v in d.items() if k in names}
         if "num_experts" in d and "num_local_experts" not in d:
@@ -126,6 +137,42 @@ class ModelConfig:
             kw["attention_sinks"] = True
             kw["attention_bias"] = True
         return cls(**kw)
+
+
+def safetensors_shapes(path: str) -> dict:
+    """Tensor name -> shape from a safetensors file's header (8-byte little-endian length, then
+    that many bytes of JSON); no tensor data is read."""
+    with open(path, "rb") as f:
+        n = int.from_bytes(f.read(8), "little")
+        head = json.loads(f.read(n))
+    return {k: tuple(v["shape"]) for k, v in head.items() if k != "__metadata__"}
+
+
+def mekusun_config(d: dict, shapes: Optional[dict] = None) -> ModelConfig:
+    """A Mekusun ``config.json``: every size and constant comes from the file. The generic fields
+    that the engine reads (widths, layer count, vocabulary) are filled from it; the per-layer
+    descriptions stay as ``layer_specs``. Sizes the file leaves to the tensors (the rank of the
+    delta rule's decay projection) come from ``shapes``, the checkpoint's name -> shape table."""
+    layers = [json.loads(json.dumps(l)) for l in d["layers"]]
+    for i, l in enumerate(layers):
+        if l["type"] == "general_delta" and "decay_rank" not in l["mixer"] and shapes \
+                and f"l{i}.mix.w1" in shapes:
+            l["mixer"]["decay_rank"] = int(shapes[f"l{i}.mix.w1"][0])
+    moe = [l["mlp"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "moe"]
+    att = [l["mixer"] for l in layers if l["type"] == "latent_attention"]
+    return ModelConfig(
+        model_type="mekusun", hidden_size=d["width"], vocab_size=d["vocab"], num_hidden_layers=len(layers),
+        num_attention_heads=att[0]["heads"] if att else 1, num_key_value_heads=1,
+        head_dim=(att[0]["kv_rank"] + att[0]["rot_dim"]) if att else 1,
+        intermediate_size=max([l["mlp"]["ff"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "dense"]
+                              or [0]),
+        num_local_experts=max([m["router"]["experts"] for m in moe] or [0]),
+        num_experts_per_tok=max([m["router"]["top"] for m in moe] or [0]),
+        moe_intermediate_size=max([m["expert"]["ff"] for m in moe] or [0]),
+        rms_norm_eps=d["norm"]["eps"], max_position_embeddings=d.get("max_position", 1 << 20),
+        bos_token_id=d.get("bos", 0), eos_token_id=d.get("eos", -1), layer_specs=layers,
+        embedding_scale=d.get("embedding", {}).get("scale", 1.0), logit_softcap=d.get("logit_softcap", 0.0),
+        name=d.get("name", "mekusun"))
 
 
 def _llama(name, d, ffn, L, hq, hkv, vocab=128256, **kw):

@@ -52,6 +52,11 @@ class LLMEngine:
             self.bm = HybridBlockManager(rt, nb, self.runner.num_swa_blocks, cfg.cache.block_size,
                                          self.runner.max_window, cfg.cache.enable_prefix_caching,
                                          ev_on or bool(cfg.kv_offload_config), swa_events=bool(cfg.kv_offload_config))
+        elif self.runner.stateful:
+            from .state_cache import StatefulBlockManager
+
+            self.bm = StatefulBlockManager(rt.BlockManager(nb, cfg.cache.block_size, False, False),
+                                           cfg.sched.max_num_seqs)
         else:
             self.bm = rt.BlockManager(nb, cfg.cache.block_size, cfg.cache.enable_prefix_caching,
                                       ev_on or bool(cfg.kv_offload_config))
@@ -126,7 +131,48 @@ class LLMEngine:
             from .hybrid_kv import HybridTables
 
             return HybridTables(full, {sr.req.seq_id: self.bm.block_table_swa(sr.req.seq_id) for sr in so.all()})
+        if self.runner.stateful:
+            from .state_cache import SlotTables
+
+            return SlotTables(full, {sr.req.seq_id: self.bm.state_slot(sr.req.seq_id) for sr in so.all()})
         return full
+
+    # ------------------------------------------------------------ given steps (trace replay)
+    def forced_step(self, entries: list, end: list) -> Optional[torch.Tensor]:
+        """Run exactly the tokens a caller brings, through the scheduler's admission, the block /
+        state manager and the runner's step, sampling nothing. ``entries``: (request id, its next
+        tokens, places among them whose logits are wanted); a request is admitted at its first
+        entry and may skip steps. ``end``: request ids finished after this step (their pages and
+        state slot go back). Returns fp32 logits [wanted, vocab] in the order of the entries and
+        their places, or None."""
+        if self._pending is not None:
+            self.drain()
+        items = []
+        for rid, toks, _ in entries:
+            r = self.sched.requests.get(rid)
+            if r is None:
+                r = Request(rid, list(toks), SamplingParams(max_tokens=1, ignore_eos=True))
+                self.sched.add_request(r)
+            else:
+                r.prompt_token_ids.extend(toks)
+            items.append((r, len(toks)))
+        so = self.sched.schedule_given(items)
+        # rows of the step's token layout: decodes first, then the prefill portions
+        base, off = {}, len(so.decodes)
+        for i, sr in enumerate(so.decodes):
+            base[sr.req.request_id] = i
+        for sr in so.prefills:
+            base[sr.req.request_id] = off
+            off += sr.num_new_tokens
+        rows = [base[rid] + int(w) for rid, toks, want in entries for w in want]
+        logits = None
+        if not so.empty:
+            logits = self.runner.forward_logits(so, self.block_tables(so), rows)
+            self.sched.update(so, {})
+            self.step_count += 1
+        for rid in end:
+            self.sched.finish_given(rid)
+        return logits
 
     def step(self) -> list[RequestOutput]:
         # asleep, or woken from level 2 with the trainer's weights not yet sent:

@@ -38,7 +38,7 @@ from llmd_amd.parallel.comm import tp_broadcast_plan, tp_min_int
 from llmd_amd.parallel.state import get_state
 from llmd_amd.utils import markers
 
-from .attn_meta import AttnMeta
+from .attn_meta import AttnMeta, SeqMeta
 from .config import EngineConfig
 from .scheduler import ScheduledReq, SchedulerOutput
 
@@ -116,11 +116,21 @@ class ModelRunner:
         from llmd_amd.parallel import eplb
 
         eplb.configure(cfg.parallel.enable_eplb, cfg.parallel.eplb_config)
-        self.model = build_model(self.mc, device=self.device, max_pos=self.max_model_len + 1)
+        dts = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "auto": torch.bfloat16,
+               "float32": torch.float32, "fp32": torch.float32}
+        if cfg.dtype not in dts:
+            raise ValueError(f"unsupported --dtype {cfg.dtype}")
+        self.dtype = dts[cfg.dtype]
+        if self.dtype == torch.float32:  # true 32-bit matrix products
+            torch.backends.cuda.matmul.allow_tf32 = False
+            torch.backends.cudnn.allow_tf32 = False
+        self.model = build_model(self.mc, device=self.device, max_pos=self.max_model_len + 1, dtype=self.dtype)
         if cfg.load_format in ("safetensors", "auto") and cfg.weights_path:
             from llmd_amd.models.loader import load_weights
 
             load_weights(self.model, cfg.weights_path)
+        if hasattr(self.model, "finalize"):  # constants derived from the weights
+            self.model.finalize()
         if cfg.quantization == "fp8":
             from llmd_amd.models.layers import quantize_fp8
 
@@ -137,12 +147,25 @@ class ModelRunner:
             torch.cuda.synchronize()
         log.info("model %s built in %.1fs", self.mc.name, time.time() - t0)
         attn = self.model.attention_layers()
-        self.Hkv, self.D, self.L = attn[0].Hkv, attn[0].D, len(attn)
-        self.Hq = attn[0].Hq
+        self.L = len(attn)
+        self.Hkv, self.D, self.Hq = (attn[0].Hkv, attn[0].D, attn[0].Hq) if attn else (1, 1, 1)
         # cache geometry per layer: (planes, heads, dim) - K/V planes of GQA heads,
         # or one latent row per token for MLA
         self.kv_spec = self.model.kv_spec() if hasattr(self.model, "kv_spec") else (2, self.Hkv, self.D)
+        # per-layer stacks: every attention layer has its own geometry and its own pool tensor
+        self.kv_specs = self.model.kv_specs() if hasattr(self.model, "kv_specs") else None
         self.is_mla = bool(getattr(self.model, "needs_mla_rows", False))
+        # layers with per-sequence recurrent state: slots in engine/state_cache.py; steps are
+        # described per sequence (AttnMeta.seq)
+        self.stateful = bool(getattr(self.model, "stateful", False))
+        self.state_pool = None
+        if self.stateful:
+            from .state_cache import StatePool
+
+            if cfg.kv_transfer_config or cfg.kv_offload_config or cfg.enable_lora:
+                raise ValueError("stateful models run without KV transfer, KV offload and LoRA")
+            cfg.cache.enable_prefix_caching = False
+            self.state_pool = StatePool(self.model.state_layers(), cfg.sched.max_num_seqs, self.device)
         # KV storage dtype (vLLM --kv-cache-dtype): bf16 or OCP fp8
         # e4m3fn (gfx950 native) with per-layer dequant scales (k_scale/v_scale,
         # 1.0 unless the checkpoint carries calibrated ones).
@@ -159,8 +182,9 @@ class ModelRunner:
         G = self.Hq // self.Hkv
         self.max_window = max((a.window for a in attn if a.window), default=0)
         self.cascade_ok = (cfg.cache.shared_prefix_decode and cfg.cache.enable_prefix_caching and not self.is_mla
-                           and G <= 16 and 16 % G == 0)
-        self.casc_variant = ops.cascade_variant(G, self.D, self.bs, self.kv_dtype != torch.bfloat16)
+                           and not self.stateful and G <= 16 and 16 % G == 0)
+        self.casc_variant = ops.cascade_variant(G, self.D, self.bs, self.kv_dtype != torch.bfloat16) \
+            if self.cascade_ok else None
         self.cascade_ok = self.cascade_ok and self.casc_variant is not None
         self.casc_work = max(16, -(-512 // self.Hkv))  # prefix work units: ~2 workgroups per CU over kv heads
         self.casc_slots = 16                           # prefix partial slots per sequence
@@ -241,7 +265,7 @@ class ModelRunner:
         (vLLM's default); off with --disable-hybrid-kv-cache-manager. kvx P/D and the
         tiered offload move / store both pools."""
         flag = self.cfg.cache.hybrid_kv_cache_manager
-        if not self.swa_layers or not self.full_layers or self.is_mla or flag is False:
+        if not self.swa_layers or not self.full_layers or self.is_mla or self.stateful or flag is False:
             return False
         if self.cfg.parallel.enable_dbo:
             return False  # dual-batch graphs carry one set of tables
@@ -254,8 +278,15 @@ class ModelRunner:
     def block_bytes(self) -> int:
         """Bytes of one block of the main pool (all layers, or the full-attention
         layers of a hybrid cache)."""
+        if self.kv_specs is not None:
+            es = torch.empty(0, dtype=self._kv_store_dtype()).element_size()
+            return max(1, sum(p * h * self.bs * d * es for p, h, d in self.kv_specs))
         n = len(self.full_layers) if self.hybrid else self.L
         return n * self.layer_bytes_per_block()
+
+    def _kv_store_dtype(self):
+        """Per-layer stacks cache in the activation type (float32 runs keep exact keys)."""
+        return self.dtype if self.kv_dtype == torch.bfloat16 else self.kv_dtype
 
     def swa_block_bytes(self) -> int:
         return len(self.swa_layers) * self.layer_bytes_per_block()
@@ -275,6 +306,12 @@ class ModelRunner:
                 and os.environ.get("LLMD_KV_VMM", "1") != "0")
 
     def _alloc_cache(self, num_blocks: int, scratch: bool = False) -> torch.Tensor:
+        if self.kv_specs is not None:  # one pool tensor per attention layer, each with its own row size
+            kv = [torch.empty((num_blocks, p, h, self.bs, d), dtype=self._kv_store_dtype(), device=self.device)
+                  for p, h, d in self.kv_specs]
+            self.vmm = None
+            self._bind(kv)
+            return kv
         planes, heads, dim = self.kv_spec
         shape = (len(self.full_layers) if self.hybrid else self.L, num_blocks, planes, heads, self.bs, dim)
         if self.hybrid:
@@ -375,6 +412,15 @@ class ModelRunner:
         return self.num_blocks
 
     def _dummy_prefill(self, T: int, nblocks: int):
+        if self.stateful:  # one sequence of T tokens over the scratch blocks, state slot 0
+            bt = np.zeros((1, self.width), dtype=np.int32)
+            nb = math.ceil(T / self.bs)
+            bt[0, :nb] = np.arange(nb)
+            pl = {"graph": False, "nd": 0, "ids": [0] * T, "pos": list(range(T)), "slots": list(range(T)),
+                  "d_bt": np.zeros((0, self.width), np.int32), "d_len": np.zeros(0, np.int32), "p_ql": [T],
+                  "p_ctx": [T], "p_bt": bt, "rows": [T - 1], "seq": ([0], [0])}
+            self.model.compute_logits(self._run_eager(pl)[-1:])
+            return
         nseq = max(1, math.ceil(T / self.bs))
         ql = [min(self.bs, T - i * self.bs) for i in range(nseq)]
         ql = [q for q in ql if q > 0]
@@ -561,6 +607,10 @@ class ModelRunner:
               "d_len": d_len, "p_ql": p_ql, "p_ctx": p_ctx, "p_bt": p_bt, "rows": rows}
         if self.hybrid:
             pl["swa"] = self._group_tables(so, block_tables.swa)
+        if self.stateful:  # state slot and "continues earlier state" flag per sequence, step order
+            pl["graph"] = False
+            pl["seq"] = ([block_tables.slots[sr.req.seq_id] for sr in so.all()],
+                         [int(sr.start > 0) for sr in so.all()])
         if self.lora is not None:
             lo = [sr.req.lora_id for sr in so.decodes]
             for sr in so.prefills:
@@ -713,6 +763,14 @@ class ModelRunner:
             host = host.pin_memory()
         hd = host.to(dev, non_blocking=True)
         meta = AttnMeta(num_tokens=T, positions=hd[1], slot_mapping=hd[2], num_decode=nd)
+        if pl.get("seq") is not None:
+            meta.num_prefill_tokens = sum(p_ql)
+            meta.seq = self._seq_meta(pl)
+            ids = hd[0]
+            if pl.get("gather") is not None:  # async: decode inputs sampled by the step still in flight
+                dst, src, prev_ids = pl["gather"]
+                ids.index_copy_(0, dst, prev_ids.index_select(0, src).to(ids.dtype))
+            return ids, meta
         if nd:
             meta.d_block_tables = torch.from_numpy(d_bt).to(dev, non_blocking=True)
             meta.d_seq_lens = torch.from_numpy(d_len).to(dev, non_blocking=True)
@@ -748,6 +806,42 @@ class ModelRunner:
             dst, src, prev_ids = pl["gather"]
             ids.index_copy_(0, dst, prev_ids.index_select(0, src).to(ids.dtype))
         return ids, meta
+
+    def _seq_meta(self, pl: dict) -> SeqMeta:
+        """The step per sequence: decodes (one token each) first, then the prefill portions."""
+        nd, p_ql, p_ctx = pl["nd"], pl["p_ql"], pl["p_ctx"]
+        dev = self.device
+        slots, init = pl["seq"]
+        ql = np.asarray([1] * nd + list(p_ql), dtype=np.int64)
+        n = len(ql)
+        start = np.zeros(n + 1, dtype=np.int32)
+        start[1:] = np.cumsum(ql)
+        row_seq = np.repeat(np.arange(n, dtype=np.int32), ql)
+        row_len = (np.asarray(pl["pos"], dtype=np.int64) + 1).astype(np.int32)
+        tables = np.concatenate([pl["d_bt"], pl["p_bt"]]) if n else np.zeros((0, self.width), np.int32)
+        small = torch.from_numpy(np.concatenate([start, np.asarray(slots, np.int32), np.asarray(init, np.int32),
+                                                 row_seq, row_len]))
+        if self.is_gpu:
+            small = small.pin_memory()
+        sd = small.to(dev, non_blocking=True)
+        T = len(row_seq)
+        o = np.cumsum([0, n + 1, n, n, T, T])
+        return SeqMeta(num_seqs=n, seq_start=sd[o[0]:o[1]], seq_slot=sd[o[1]:o[2]], seq_init=sd[o[2]:o[3]],
+                       row_seq=sd[o[3]:o[4]], row_len=sd[o[4]:o[5]],
+                       tables=torch.from_numpy(np.ascontiguousarray(tables)).to(dev, non_blocking=True),
+                       max_len=int(row_len.max()) if T else 0)
+
+    @torch.no_grad()
+    def forward_logits(self, so: SchedulerOutput, block_tables: dict, rows: list[int]):
+        """One step over ``so`` that samples nothing: fp32 logits of the step's token rows ``rows``
+        (decodes first, then the prefill portions in order), or None when none are asked for."""
+        pl, _ = self.plan(so, block_tables)
+        pl["graph"] = False
+        pl["rows"] = list(rows)
+        if self.tp_size > 1:
+            tp_broadcast_plan(pl)
+        logits = self.run_plan(pl)
+        return None if logits is None else logits.float()
 
     def _cascade_plan(self, d_bt, d_len, max_work=None):
         """Shared-prefix decode plan for this step's decode rows, or None."""
@@ -868,7 +962,7 @@ class ModelRunner:
 
     @torch.no_grad()
     def capture_graphs(self):
-        if not self.is_gpu or self.cfg.enforce_eager:
+        if not self.is_gpu or self.cfg.enforce_eager or self.stateful:
             return
         maxb = min(self.cfg.cuda_graph_max_bs, self.cfg.sched.max_num_seqs)
         buckets = []

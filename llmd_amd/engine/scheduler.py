@@ -368,6 +368,45 @@ class Scheduler:
         self._align_tokens(out)
         return out
 
+    def schedule_given(self, items: list) -> SchedulerOutput:
+        """A step whose portions the caller fixes: ``items`` = (request, number of its next
+        tokens). Waiting requests are admitted (pages and, for stateful models, a state slot);
+        nothing is preempted and nothing trimmed - a step that does not fit raises."""
+        out = SchedulerOutput()
+        for r, n in items:
+            if n <= 0:
+                continue
+            if r not in self.running:
+                if len(self.running) >= self.sc.max_num_seqs:
+                    raise RuntimeError(f"more than max_num_seqs={self.sc.max_num_seqs} live requests")
+                if not self.waiting.remove(r):
+                    raise ValueError(f"request {r.request_id} is neither waiting nor running")
+                if not self.bm.has_seq(r.seq_id):
+                    r.num_computed_tokens = self.bm.acquire(r.seq_id, self._tokens(r), r.cache_extra)
+                r.status = Status.RUNNING
+                if r.first_scheduled_time is None:
+                    r.first_scheduled_time = time.monotonic()
+                self.running.append(r)
+            if r.num_computed_tokens + n > r.num_tokens:
+                raise ValueError(f"request {r.request_id}: {n} tokens asked, "
+                                 f"{r.num_tokens - r.num_computed_tokens} left")
+            if not self.bm.grow(r.seq_id, r.num_computed_tokens + n):
+                raise RuntimeError(f"request {r.request_id}: no room for {r.num_computed_tokens + n} tokens")
+            sr = ScheduledReq(r, n, r.num_computed_tokens)
+            (out.decodes if sr.is_decode else out.prefills).append(sr)
+        return out
+
+    def finish_given(self, request_id: str) -> None:
+        """End a request driven through ``schedule_given``: its pages and slot go back."""
+        r = self.requests.get(request_id)
+        if r is None or r.status.finished:
+            return
+        if r in self.running:
+            self._finish_running(r, Status.FINISHED_LENGTH)
+        else:
+            self.waiting.remove(r)
+            self._finish(r, Status.FINISHED_LENGTH)
+
     def _reload_cannot_fit(self, r, cached: int, budget: int) -> bool:
         """True when the pool cannot hold this request's first chunk even after a
         tier reload (the blocks it holds now plus the free ones): reloading host /

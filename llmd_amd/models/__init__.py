@@ -1,6 +1,8 @@
 """Model registry: HF ``model_type`` -> implementation."""
 from __future__ import annotations
 
+import torch
+
 from llmd_amd.engine.config import ModelConfig
 
 
@@ -30,8 +32,17 @@ def model_class(cfg: ModelConfig):
         from .moe_llama import MoELlamaForCausalLM
 
         return MoELlamaForCausalLM
+    if t == "mekusun":
+        from .mekusun import MekusunForCausalLM
+
+        return MekusunForCausalLM
     raise ValueError(f"unsupported model_type {t!r}")
 
 
-def build_model(cfg: ModelConfig, device="cuda", max_pos: int = 32768):
-    return model_class(cfg)(cfg, device=device, max_pos=max_pos)
+def build_model(cfg: ModelConfig, device="cuda", max_pos: int = 32768, dtype=None):
+    cls = model_class(cfg)
+    if dtype is not None and dtype != torch.bfloat16:
+        if not getattr(cls, "supports_float32", False):
+            raise ValueError(f"{cfg.model_type} runs in bfloat16 only")
+        return cls(cfg, device=device, max_pos=max_pos, dtype=dtype)
+    return cls(cfg, device=device, max_pos=max_pos)

@@ -1,0 +1,200 @@
+"""Sequence mixers and feed-forwards for per-layer stacks (models/mekusun.py): every size and
+constant is an argument, so another stack can reuse them.
+
+* ``LatentAttention``  - attention over a low-rank latent cache, any (heads, unrotated dim,
+  rotated dim, value dim, latent rank); weight-absorbed, so the paged cache holds one row
+  [latent | rotated shared key] per token (the fixed-size DeepSeek form is models/deepseek.py).
+* ``Mamba1Mixer``      - selective state-space scan with a short causal convolution.
+* ``GeneralDeltaMixer``- generalized delta rule with per-channel decay and removal rate.
+* ``ActMLP`` / ``PlainMoE`` - ungated feed-forwards (xIELU dense; erf-GELU experts with a
+  biased fp32 router and softmax over the chosen logits).
+
+Recurrent state lives in the engine's state pool (engine/state_cache.py): a mixer with
+``state_shapes()`` gets its per-slot tensors through ``bind_state``; the step's
+``AttnMeta.seq`` says which slot each run of tokens continues. Matrix products go to the
+vendor GEMM through ``ops.linear``; everything between them runs in the kernels of
+``ops.seqmix`` (fp32 where the recurrences, norms and scores need it).
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+from llmd_amd.engine.attn_meta import AttnMeta
+from llmd_amd.ops import seqmix as sm
+
+from .layers import ColumnLinear, _init_weight
+
+
+def _param(shape, device, dtype, std=0.02, fill=None):
+    t = torch.empty(shape, device=device, dtype=dtype)
+    if fill is None:
+        _init_weight(t, std)
+    else:
+        t.fill_(fill)
+    return torch.nn.Parameter(t, requires_grad=False)
+
+
+def rope_table(dims: int, base: float, max_pos: int, device) -> torch.Tensor:
+    """[max_pos, dims] fp32 = [cos(p f_i) | sin(p f_i)], f_i = base^(-2i/dims), angles in fp64."""
+    half = dims // 2
+    f = torch.tensor(base, dtype=torch.float64) ** (-2.0 * torch.arange(half, dtype=torch.float64) / dims)
+    a = torch.arange(max_pos, dtype=torch.float64)[:, None] * f[None]
+    return torch.cat([a.cos(), a.sin()], -1).float().to(device)
+
+
+class LatentAttention(torch.nn.Module):
+    is_latent = True
+
+    def __init__(self, d_model, heads, dim, rot_dim, vdim, kv_rank, scale, rot_dims, rot_base, eps, max_pos,
+                 device, dtype):
+        super().__init__()
+        if rot_dims > rot_dim or rot_dims % 2:
+            raise ValueError(f"rotary dims {rot_dims} do not fit the rotated part {rot_dim}")
+        self.H, self.dn, self.dr, self.dv, self.R = heads, dim, rot_dim, vdim, kv_rank
+        self.scale, self.rot_dims, self.eps = float(scale), rot_dims, eps
+        self.q = ColumnLinear(d_model, heads * (dim + rot_dim), shard=False, device=device, dtype=dtype)
+        self.dkv = ColumnLinear(d_model, kv_rank + rot_dim, shard=False, device=device, dtype=dtype)
+        self.dkv_norm = _param((kv_rank,), device, dtype, fill=1.0)
+        self.uk = _param((heads * dim, kv_rank), device, dtype)
+        self.uv = _param((heads * vdim, kv_rank), device, dtype)
+        self.o = ColumnLinear(heads * vdim, d_model, shard=False, device=device, dtype=dtype)
+        self.register_buffer("cos_sin", rope_table(rot_dims, rot_base, max_pos, device), persistent=False)
+        self.cache = None
+        # what the runner's generic bookkeeping reads
+        self.Hq, self.Hkv, self.D, self.window, self.sinks = heads, 1, kv_rank + rot_dim, 0, None
+
+    def kv_spec(self):
+        return 1, 1, self.R + self.dr  # (planes, heads, dim): one latent row per token
+
+    def bind_cache(self, kv_layer):
+        """kv_layer [blocks, 1, 1, bs, R + dr] -> [blocks, bs, R + dr]."""
+        self.cache = kv_layer[:, 0, 0]
+
+    def forward(self, h, meta: AttnMeta):
+        T, H, R, dn, dr = h.shape[0], self.H, self.R, self.dn, self.dr
+        s = meta.seq
+        q = self.q(h)
+        kv = self.dkv(h)
+        q_abs = torch.empty(T, H, R + dr, dtype=h.dtype, device=h.device)
+        sm.latent_rope_cache(q, kv, self.dkv_norm, self.eps, meta.positions, self.cos_sin, H, dn, dr,
+                             self.rot_dims, R, meta.slot_mapping, self.cache, q_abs)
+        # absorb W_uk into the query: scores against the latent itself
+        qn = q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1)                       # [H, T, dn]
+        q_abs[:, :, :R].copy_(torch.bmm(qn, self.uk.view(H, dn, R)).transpose(0, 1))
+        o_lat = sm.latent_attention(q_abs, self.cache, s.tables, s.row_seq, s.row_len, self.scale, R)
+        o = torch.bmm(o_lat.transpose(0, 1), self.uv.view(H, self.dv, R).transpose(1, 2))  # [H, T, dv]
+        return self.o(o.transpose(0, 1).reshape(T, H * self.dv))
+
+
+class Mamba1Mixer(torch.nn.Module):
+    def __init__(self, d_model, inner, state, dt_rank, taps, device, dtype):
+        super().__init__()
+        self.C, self.N, self.R, self.taps = inner, state, dt_rank, taps
+        self.dtype = dtype
+        self.in_proj = ColumnLinear(d_model, 2 * inner, shard=False, device=device, dtype=dtype)
+        self.conv = _param((inner, taps), device, dtype, std=0.2)
+        self.conv_b = _param((inner,), device, dtype, fill=0.0)
+        self.x_proj = ColumnLinear(inner, dt_rank + 2 * state, shard=False, device=device, dtype=dtype)
+        self.dt_proj = ColumnLinear(dt_rank, inner, shard=False, device=device, dtype=dtype)
+        self.dt_b = _param((inner,), device, dtype, fill=0.0)
+        self.A_log = _param((inner, state), device, dtype, fill=0.0)
+        self.D = _param((inner,), device, dtype, fill=1.0)
+        self.o = ColumnLinear(inner, d_model, shard=False, device=device, dtype=dtype)
+        self.A = None
+        self.conv_state = self.ssm_state = None
+
+    def finalize(self):
+        """After the weights are loaded: A = -exp(A_log) once, in fp32."""
+        self.A = -torch.exp(self.A_log.data.float())
+
+    def state_shapes(self):
+        return [((max(self.taps - 1, 1), self.C), self.dtype), ((self.C, self.N), torch.float32)]
+
+    def bind_state(self, tensors):
+        self.conv_state, self.ssm_state = tensors
+
+    def forward(self, h, meta: AttnMeta):
+        s = meta.seq
+        xz = self.in_proj(h)
+        xc = sm.causal_conv_silu(xz, self.C, self.conv, self.conv_b, self.conv_state, s.seq_start, s.seq_slot,
+                                 s.seq_init)
+        bc = self.x_proj(xc)
+        dt_raw = self.dt_proj(bc[:, :self.R])
+        y = sm.selective_scan(xc, dt_raw, self.dt_b, self.A, bc, self.R, self.N, self.D, xz, self.C,
+                              self.ssm_state, s.seq_start, s.seq_slot, s.seq_init)
+        return self.o(y)
+
+
+class GeneralDeltaMixer(torch.nn.Module):
+    def __init__(self, d_model, heads, dim, decay_rank, eps, device, dtype):
+        super().__init__()
+        self.H, self.d, self.eps, self.wr = heads, dim, eps, decay_rank
+        HD = heads * dim
+        # one projection of the layer input: [r | k | v | g | a | decay low-rank]
+        self.proj = ColumnLinear(d_model, 5 * HD + decay_rank, shard=False, device=device, dtype=dtype)
+        self.a_b = _param((HD,), device, dtype, fill=0.0)
+        self.w2 = ColumnLinear(decay_rank, HD, shard=False, device=device, dtype=dtype)
+        self.w0 = _param((HD,), device, dtype, fill=0.0)
+        self.norm = _param((HD,), device, dtype, fill=1.0)
+        self.o = ColumnLinear(HD, d_model, shard=False, device=device, dtype=dtype)
+        self.state = None
+
+    def state_shapes(self):
+        return [((self.H, self.d, self.d), torch.float32)]
+
+    def bind_state(self, tensors):
+        (self.state,) = tensors
+
+    def forward(self, h, meta: AttnMeta):
+        s = meta.seq
+        HD = self.H * self.d
+        p = self.proj(h)
+        wl = self.w2(torch.tanh(p[:, 5 * HD:]))
+        y = sm.gdelta_scan(p, wl, self.w0, self.a_b, self.norm, self.eps, self.H, self.d, self.state,
+                           s.seq_start, s.seq_slot, s.seq_init)
+        return self.o(y)
+
+
+class ActMLP(torch.nn.Module):
+    """W_down xielu(W_up h): the activation's two numbers are stored raw (``act``); their
+    softplus forms are taken once after loading."""
+
+    def __init__(self, d_model, ff, device, dtype):
+        super().__init__()
+        self.up = ColumnLinear(d_model, ff, shard=False, device=device, dtype=dtype)
+        self.down = ColumnLinear(ff, d_model, shard=False, device=device, dtype=dtype)
+        self.act = _param((2,), device, dtype, fill=0.0)
+        self.ap = self.aq = None
+
+    def finalize(self):
+        p, q = self.act.data.double().cpu().tolist()
+        sp = lambda v: max(v, 0.0) + math.log1p(math.exp(-abs(v)))  # noqa: E731
+        self.ap, self.aq = sp(p), 0.5 + sp(q)
+
+    def forward(self, h):
+        return self.down(sm.xielu(self.up(h), self.ap, self.aq))
+
+
+class PlainMoE(torch.nn.Module):
+    """Ungated experts W_down gelu(W_up h); router logits W_r h + b in fp32, the ``top`` largest
+    chosen, weights = softmax over the chosen logits."""
+
+    def __init__(self, d_model, ff, experts, top, device, dtype):
+        super().__init__()
+        self.E, self.k = experts, top
+        self.router = _param((experts, d_model), device, dtype)
+        self.router_b = _param((experts,), device, dtype, fill=0.0)
+        self.w1 = _param((experts, ff, d_model), device, dtype)
+        self.w2 = _param((experts, d_model, ff), device, dtype)
+        self.router32 = self.router_b32 = None
+
+    def finalize(self):
+        self.router32, self.router_b32 = self.router.data.float(), self.router_b.data.float()
+
+    def forward(self, h):
+        logits = F.linear(h.float(), self.router32, self.router_b32)
+        ids, w = sm.moe_route(logits, self.k)
+        return sm.moe_ffn(h, ids, w, self.w1, self.w2)

@@ -1,0 +1,187 @@
+"""Ops of per-layer ("sequence mixer") stacks: latent attention of any size, the selective
+scan, the generalized delta rule, zero-centred norms with layer scale, depth averaging, plain
+(ungated) expert feed-forwards.
+
+GPU tensors go to the ``llmd_amd._C_seqmix`` library (csrc/seqmix/*.hip, built on its own so a
+model that needs only these kernels compiles only these); it is templated on the activation
+type, bfloat16 or float32, and keeps in fp32 what the recurrences, norms, scores and the
+residual need. CPU tensors use ``seqmix_ref``. A missing library on a GPU host raises.
+
+Step layout (engine/attn_meta.py SeqMeta): the step's tokens are the sequences' runs back to
+back; ``seq_start`` [n+1] bounds them, ``seq_slot`` [n] is each sequence's state slot and
+``seq_init`` [n] says whether the slot holds the sequence's earlier state (0: start from zero).
+"""
+from __future__ import annotations
+
+import importlib
+import os
+
+import torch
+
+from . import seqmix_ref as ref
+
+_LIB = None
+
+
+def native():
+    global _LIB
+    if _LIB is None:
+        try:
+            _LIB = importlib.import_module("llmd_amd._C_seqmix")
+        except ImportError as e:
+            if os.environ.get("LLMD_AUTOBUILD", "1") != "1":
+                raise RuntimeError(f"llmd_amd._C_seqmix HIP extension not built: {e}") from e
+            from llmd_amd.build import build_seqmix
+
+            build_seqmix()
+            _LIB = importlib.import_module("llmd_amd._C_seqmix")
+    return _LIB
+
+
+def embed_scale(ids, table, scale: float, hist):
+    """hist[0] = hist[1] = table[ids] * scale (fp32): the embedding output and the first layer's
+    working residual."""
+    if not ids.is_cuda:
+        return ref.embed_scale(ids, table, scale, hist)
+    native().embed_scale(ids, table, float(scale), hist)
+
+
+def zc_norm(x, w, eps: float, out_dtype):
+    """RMS norm of the fp32 residual with a weight stored around zero: x / rms(x) * (1 + w)."""
+    if not x.is_cuda:
+        return ref.zc_norm(x, w, eps, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    native().zc_norm(x, w, float(eps), out)
+    return out
+
+
+def add_post_norm(y, w_post, ls, x, eps: float, next_w=None, out_dtype=None):
+    """x += ls * zc_norm(y, w_post) on the fp32 residual, in place; with ``next_w`` also returns
+    zc_norm(x, next_w), the next sublayer's input, from the same pass."""
+    if not x.is_cuda:
+        return ref.add_post_norm(y, w_post, ls, x, eps, next_w, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device) if next_w is not None else None
+    native().add_post_norm(y, w_post, ls, x, float(eps), next_w, out)
+    return out
+
+
+def depth_avg_norm(hist, n: int, coef, dst: int, norm_w, eps: float, out_dtype):
+    """hist[dst] = sum_{j<n} coef[j] * hist[j] (fp32) and the zero-centred norm of that sum."""
+    if not hist.is_cuda:
+        return ref.depth_avg_norm(hist, n, coef, dst, norm_w, eps, out_dtype)
+    out = torch.empty(hist.shape[1:], dtype=out_dtype, device=hist.device)
+    native().depth_avg_norm(hist, int(n), coef, int(dst), norm_w, float(eps), out)
+    return out
+
+
+def latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache, q_abs):
+    """Rotate the rotary part of q into ``q_abs[..., R:]``; write [norm(kv[:, :R]) | rot(kv[:, R:])]
+    to the paged latent cache at ``slots`` (-1: no write). cos_sin [max_pos, rot_dims] fp32."""
+    if not q.is_cuda:
+        return ref.latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache,
+                                     q_abs)
+    native().latent_rope_cache(q, kv, norm_w, float(eps), positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache,
+                               q_abs)
+
+
+def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: int, max_len: int = 0):
+    """Causal softmax attention of absorbed queries [T, H, R + dr] over the paged latent cache
+    [blocks, bs, R + dr]; row t sees the first row_len[t] keys of sequence row_seq[t].
+    Returns the latent outputs [T, H, R]."""
+    T, H, _ = q_abs.shape
+    out = torch.empty(T, H, R, dtype=q_abs.dtype, device=q_abs.device)
+    if not q_abs.is_cuda:
+        return ref.latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out)
+    native().latent_attention(q_abs, cache, tables, row_seq, row_len, float(scale), R, out)
+    return out
+
+
+def causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init):
+    """Per-channel causal convolution + SiLU over the first C columns of xz, continuing from each
+    sequence's last taps-1 inputs in ``conv_state`` [slots, taps-1, C] (updated)."""
+    out = torch.empty(xz.shape[0], C, dtype=xz.dtype, device=xz.device)
+    if not xz.is_cuda:
+        return ref.causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init, out)
+    native().causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init, out)
+    return out
+
+
+def selective_scan(xc, dt_raw, dt_bias, A, bc, R, N, D, xz, C, state, seq_start, seq_slot, seq_init):
+    """S <- exp(dt A) S + dt x B; y = S C + D x; y * silu(z). dt = softplus(dt_raw + dt_bias);
+    B, C are columns [R, R+N) and [R+N, R+2N) of ``bc``; z the columns [C, 2C) of xz. ``state``
+    [slots, C, N] fp32 is continued and updated."""
+    out = torch.empty_like(xc)
+    if not xc.is_cuda:
+        return ref.selective_scan(xc, dt_raw, dt_bias, A, bc, R, N, D, xz, C, state, seq_start, seq_slot, seq_init,
+                                  out)
+    native().selective_scan(xc, dt_raw, dt_bias, A, bc, R, N, D, xz, C, state, seq_start, seq_slot, seq_init, out)
+    return out
+
+
+def gdelta_scan(proj, wl, w0, a_b, norm_w, eps, H, d, state, seq_start, seq_slot, seq_init):
+    """Generalized delta rule over ``proj`` = [r | k | v | g | a] (H*d columns each) with decay
+    logits ``wl``: S <- diag(w) S - (a u)(u^T S) + k v^T, o = S^T r, then per-head RMS norm,
+    ``norm_w`` and the sigmoid gate. ``state`` [slots, H, d, d] fp32."""
+    out = torch.empty(proj.shape[0], H * d, dtype=proj.dtype, device=proj.device)
+    if not proj.is_cuda:
+        return ref.gdelta_scan(proj, wl, w0, a_b, norm_w, eps, H, d, state, seq_start, seq_slot, seq_init, out)
+    native().gdelta_scan(proj, wl, w0, a_b, norm_w, float(eps), H, d, state, seq_start, seq_slot, seq_init, out)
+    return out
+
+
+def xielu(z, ap: float, aq: float):
+    """z > 0: ap z^2 + z/2; else aq (exp(z) - 1 - z) + z/2."""
+    if not z.is_cuda:
+        return ref.xielu(z, ap, aq)
+    out = torch.empty_like(z)
+    native().xielu(z, float(ap), float(aq), out)
+    return out
+
+
+def moe_route(logits, k: int):
+    """Top-k of fp32 router logits (ties: lower index) and the softmax over the chosen ones."""
+    if not logits.is_cuda:
+        return ref.moe_route(logits, k)
+    T = logits.shape[0]
+    ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+    w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    native().moe_route(logits, k, ids, w)
+    return ids, w
+
+
+MOE_TILE = 64
+
+
+def moe_ffn(h, ids, w, w1, w2):
+    """sum_j w[t, j] * W2[e] gelu(W1[e] h_t), e = ids[t, j]: ungated experts with the exact (erf)
+    GELU. w1 [E, F, d], w2 [E, d, F]. Rows are grouped by expert into 64-row tiles (one pass of a
+    single workgroup), two grouped GEMMs run over the tiles, and the combine sums each token's
+    rows in fp32; a row's sums do not depend on what else is in the step."""
+    if not h.is_cuda:
+        return ref.moe_ffn(h, ids, w, w1, w2)
+    C = native()
+    T, d = h.shape
+    k = ids.shape[1]
+    E, Fh, _ = w1.shape
+    n = T * k
+    max_tiles = (n + E * (MOE_TILE - 1)) // MOE_TILE + 1
+    dev = h.device
+    slot_row = torch.empty(max_tiles * MOE_TILE, dtype=torch.int32, device=dev)   # tile slot -> pair index or -1
+    tile_e = torch.empty(max_tiles, dtype=torch.int32, device=dev)                # tile -> expert or -1
+    pair_slot = torch.empty(n, dtype=torch.int32, device=dev)                      # pair -> tile slot
+    C.moe_group(ids, E, slot_row, tile_e, pair_slot)
+    a = torch.empty(max_tiles * MOE_TILE, Fh, dtype=h.dtype, device=dev)
+    y = torch.empty(max_tiles * MOE_TILE, d, dtype=h.dtype, device=dev)
+    C.moe_gemm(h, k, slot_row, tile_e, w1, a, True)
+    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, False)
+    out = torch.empty_like(h)
+    C.moe_combine(y, pair_slot, w, out)
+    return out
+
+
+def softcap_(logits, cap: float):
+    """logits <- cap * tanh(logits / cap), in place (fp32)."""
+    if not logits.is_cuda:
+        return ref.softcap_(logits, cap)
+    native().softcap(logits, float(cap))
+    return logits

@@ -1,0 +1,151 @@
+"""CPU implementations (plain torch, fp32 math) of the ops in ``llmd_amd.ops.seqmix``.
+
+They exist so that the engine, its scheduler and its state manager run in CPU CI; GPU tensors
+never come here. Arguments are the ones of the wrappers in ``seqmix.py``.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def _zc(x, w, eps):
+    x = x.float()
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + w.float())
+
+
+def embed_scale(ids, table, scale, hist):
+    x = table[ids].float() * scale
+    hist[0].copy_(x)
+    hist[1].copy_(x)
+
+
+def zc_norm(x, w, eps, out_dtype):
+    return _zc(x, w, eps).to(out_dtype)
+
+
+def add_post_norm(y, w_post, ls, x, eps, next_w, out_dtype):
+    x.add_(_zc(y, w_post, eps) * ls.float())
+    return None if next_w is None else _zc(x, next_w, eps).to(out_dtype)
+
+
+def depth_avg_norm(hist, n, coef, dst, norm_w, eps, out_dtype):
+    x = (hist[:n] * coef[:n].float().view(n, 1, 1)).sum(0)
+    hist[dst].copy_(x)
+    return _zc(x, norm_w, eps).to(out_dtype)
+
+
+def _rot(v, cs, dims):
+    half = dims // 2
+    c, s = cs[..., :half], cs[..., half:]
+    a, b = v[..., :half].float(), v[..., half:dims].float()
+    return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:].float()], -1)
+
+
+def latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache, q_abs):
+    T = q.shape[0]
+    cs = cos_sin[positions]                                  # [T, rot_dims]
+    qr = _rot(q.view(T, H, dn + dr)[..., dn:], cs[:, None], rot_dims)
+    q_abs.view(T, H, R + dr)[..., R:] = qr.to(q_abs.dtype)
+    c = kv[:, :R].float()
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    row = torch.cat([c, _rot(kv[:, R:], cs, rot_dims)], -1).to(cache.dtype)
+    ok = slots >= 0
+    cache.view(-1, R + dr)[slots[ok]] = row[ok]
+
+
+def latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out):
+    T, H, Dk = q_abs.shape
+    bs = cache.shape[1]
+    flat = cache.view(-1, Dk)
+    for t in range(T):
+        n = int(row_len[t])
+        bt = tables[int(row_seq[t])].long()
+        idx = bt[torch.arange(n) // bs] * bs + torch.arange(n) % bs
+        K = flat[idx].float()                               # [n, Dk]
+        s = (q_abs[t].float() @ K.T) * scale
+        p = torch.softmax(s, -1)
+        out[t] = (p @ K[:, :R]).to(out.dtype)
+    return out
+
+
+def causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init, out):
+    taps = w.shape[1]
+    wf, bf = w.float(), b.float()
+    for i in range(seq_slot.numel()):
+        lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
+        x = xz[lo:hi, :C].float()
+        prev = conv_state[sl].float() if int(seq_init[i]) else torch.zeros(taps - 1, C)
+        xp = torch.cat([prev, x])
+        acc = bf.expand(hi - lo, C).clone()
+        for j in range(taps):
+            acc += xp[j:j + hi - lo] * wf[:, j]
+        out[lo:hi] = F.silu(acc).to(out.dtype)
+        if taps > 1:
+            conv_state[sl] = xp[-(taps - 1):].to(conv_state.dtype)
+    return out
+
+
+def selective_scan(xc, dt_raw, dt_bias, A, bc, R, N, D, xz, C, state, seq_start, seq_slot, seq_init, out):
+    Df, bias = D.float(), dt_bias.float()
+    for i in range(seq_slot.numel()):
+        lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
+        S = state[sl].clone() if int(seq_init[i]) else torch.zeros_like(state[sl])
+        for t in range(lo, hi):
+            dt = F.softplus(dt_raw[t].float() + bias)
+            x = xc[t].float()
+            Bt, Ct = bc[t, R:R + N].float(), bc[t, R + N:R + 2 * N].float()
+            S = torch.exp(dt[:, None] * A) * S + (dt * x)[:, None] * Bt[None]
+            y = S @ Ct + Df * x
+            out[t] = (y * F.silu(xz[t, C:].float())).to(out.dtype)
+        state[sl] = S
+    return out
+
+
+DECAY_K = math.exp(-0.5)
+
+
+def gdelta_scan(proj, wl, w0, a_b, norm_w, eps, H, d, state, seq_start, seq_slot, seq_init, out):
+    HD = H * d
+    for i in range(seq_slot.numel()):
+        lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
+        S = state[sl].clone() if int(seq_init[i]) else torch.zeros_like(state[sl])
+        for t in range(lo, hi):
+            p = proj[t].float()
+            r, k, v, g, al = (p[j * HD:(j + 1) * HD].view(H, d) for j in range(5))
+            w = torch.exp(-DECAY_K * torch.sigmoid(wl[t].float() + w0.float())).view(H, d)
+            a = torch.sigmoid(al + a_b.float().view(H, d))
+            u = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+            uS = torch.einsum("hi,hij->hj", u, S)
+            S = w[:, :, None] * S - (a * u)[:, :, None] * uS[:, None] + k[:, :, None] * v[:, None]
+            o = torch.einsum("hij,hi->hj", S, r)
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+            out[t] = (o * norm_w.float().view(H, d) * torch.sigmoid(g)).reshape(HD).to(out.dtype)
+        state[sl] = S
+    return out
+
+
+def xielu(z, ap, aq):
+    zf = z.float()
+    return torch.where(zf > 0, ap * zf * zf + 0.5 * zf, aq * (torch.expm1(zf) - zf) + 0.5 * zf).to(z.dtype)
+
+
+def moe_route(logits, k):
+    top, ids = logits.float().topk(k, -1)
+    return ids.int(), torch.softmax(top, -1)
+
+
+def moe_ffn(h, ids, w, w1, w2):
+    out = torch.zeros(h.shape, dtype=torch.float32)
+    hf = h.float()
+    for e in ids.unique().tolist():
+        t, j = (ids == e).nonzero(as_tuple=True)
+        a = F.gelu((hf[t] @ w1[e].float().T).to(h.dtype).float()).to(h.dtype).float()
+        out.index_add_(0, t, (a @ w2[e].float().T) * w[t, j, None])
+    return out.to(h.dtype)
+
+
+def softcap_(logits, cap):
+    return logits.copy_(cap * torch.tanh(logits / cap))
