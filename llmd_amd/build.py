@@ -125,6 +125,37 @@ def build_ops(jobs: int = 8, verbose: bool = False, debug: bool = False) -> Path
     return out
 
 
+def build_seqmix(jobs: int = 8, verbose: bool = False) -> Path:
+    """Build ``llmd_amd/_C_seqmix``: the kernels of per-layer stacks (latent attention of any
+    size, selective scan, delta rule, zero-centred norms, ungated experts; ``csrc/seqmix``). It is a
+    library of its own so that a model that needs only these compiles only these."""
+    tinc, tlib = _torch_paths()
+    name = "_C_seqmix"
+    out_dir = BUILD / "seqmix"
+    out_dir.mkdir(parents=True, exist_ok=True)
+    src = CSRC / "seqmix"
+    deps = _headers(src)
+    hip_flags = [f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", f"-I{src}", "-ffp-contract=fast",
+                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+    cpp_flags = [
+        "-O2", "-fPIC", "-std=c++17", f"-I{ROCM}/include", f"-I{_py_inc()}",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-DTORCH_EXTENSION_NAME={name}",
+        "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=1", "-w",
+    ] + [f"-I{p}" for p in tinc]
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        futs = [ex.submit(_compile, s, [f"{ROCM}/bin/hipcc"], hip_flags, deps, out_dir)
+                for s in sorted(src.glob("*.hip"))]
+        futs.append(ex.submit(_compile, src / "bindings.cpp", ["g++"], cpp_flags, deps, out_dir))
+        objs = [f.result() for f in futs]
+    libs = [f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
+            "-lamdhip64", f"-Wl,-rpath,{tlib}"]
+    out = _link(objs, PKG / f"{name}{EXT}", libs)
+    _check_launch_stubs(out)
+    if verbose:
+        print(f"[llmd build] {out}")
+    return out
+
+
 def _check_launch_stubs(lib: Path) -> None:
     """Fail the build when a kernel's host launch stub is missing from the library: the link of a
     shared object leaves it undefined and the failure would only show at import time on the GPU box
@@ -213,6 +244,7 @@ def build_all(jobs: int | None = None, verbose: bool = True):
     build_relay(verbose)
     rt = build_runtime(jobs, verbose)
     ops = build_ops(jobs, verbose)
+    build_seqmix(jobs, verbose)
     if verbose:
         print(f"[llmd build] ok: {rt.name} {ops.name}")
     return rt, ops
@@ -224,6 +256,8 @@ if __name__ == "__main__":
         build_ops(verbose=True)
     elif what == "rt":
         build_runtime(verbose=True)
+    elif what == "seqmix":
+        build_seqmix(verbose=True)
     elif what == "relay":
         build_relay(verbose=True)
     elif what == "sanitize":

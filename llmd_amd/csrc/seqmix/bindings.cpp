@@ -1,0 +1,324 @@
+// Python bindings of the sequence-mixer op library (llmd_amd._C_seqmix). Host C++ only; the
+// kernels live in the sm_*.hip units behind extern "C" launchers. Every binding checks device,
+// dtype, contiguity and the shapes its kernel's grid assumes, so a bad call raises instead of
+// faulting the GPU. Activations are bfloat16 or float32 (f32 flag), never mixed in one call.
+#include <torch/extension.h>
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime.h>
+
+extern "C" {
+void sm_embed_scale(const int64_t*, const void*, float, float*, float*, int, int, int, hipStream_t);
+void sm_zc_norm(const float*, const void*, float, void*, int, int, int, hipStream_t);
+void sm_add_post_norm(const void*, int64_t, const void*, const void*, float*, float, const void*, void*, int, int, int,
+                      hipStream_t);
+void sm_depth_avg_norm(float*, int64_t, int, const float*, int, const void*, float, void*, int, int, int, hipStream_t);
+void sm_xielu(const void*, float, float, void*, int64_t, int, hipStream_t);
+void sm_softcap(float*, float, int64_t, hipStream_t);
+void sm_latent_rope_cache(const void*, int64_t, const void*, int64_t, const void*, float, const int64_t*, const float*,
+                          int, int, int, int, int, const int64_t*, void*, void*, int, int, hipStream_t);
+int sm_latent_attention(const void*, const void*, const int*, int, int, const int*, const int*, float, int, int, int,
+                        int, int, void*, int, hipStream_t);
+void sm_causal_conv_silu(const void*, int64_t, int, const void*, const void*, int, void*, const int*, const int*,
+                         const int*, void*, int, int, int, hipStream_t);
+int sm_selective_scan(const void*, const void*, const void*, const float*, const void*, int64_t, int, int, const void*,
+                      const void*, int64_t, int, float*, const int*, const int*, const int*, void*, int, int,
+                      hipStream_t);
+int sm_gdelta_scan(const void*, int64_t, const void*, const void*, const void*, const void*, float, int, int, float*,
+                   const int*, const int*, const int*, void*, int, int, hipStream_t);
+void sm_moe_route(const float*, int, int, int*, float*, int, hipStream_t);
+void sm_moe_group(const int*, int, int, int*, int*, int*, int, hipStream_t);
+void sm_moe_gemm(const void*, int64_t, int, const int*, const int*, const void*, int, int, void*, int, int, int,
+                 hipStream_t);
+void sm_moe_combine(const void*, const int*, const float*, int, int, void*, int, int, hipStream_t);
+}
+
+namespace {
+
+using torch::Tensor;
+
+std::optional<c10::DeviceIndex> dev_of(const Tensor& t) {
+  if (t.is_cuda()) return t.get_device();
+  return std::nullopt;
+}
+
+hipStream_t cur() { return c10::hip::getCurrentHIPStream().stream(); }
+
+bool act_ok(const Tensor& t) { return t.scalar_type() == torch::kBFloat16 || t.scalar_type() == torch::kFloat32; }
+int is_f32(const Tensor& t) { return t.scalar_type() == torch::kFloat32 ? 1 : 0; }
+
+#define CHECK_ACT(t, like) \
+  TORCH_CHECK((t).is_cuda() && (t).scalar_type() == (like).scalar_type(), #t ": device tensor of the activation type")
+#define CHECK_I32(t) TORCH_CHECK((t).is_cuda() && (t).scalar_type() == torch::kInt32 && (t).is_contiguous(), #t ": int32")
+#define CHECK_F32(t) TORCH_CHECK((t).is_cuda() && (t).scalar_type() == torch::kFloat32 && (t).is_contiguous(), #t ": fp32")
+
+void check_seq(const Tensor& seq_start, const Tensor& seq_slot, const Tensor& seq_init, int64_t slots) {
+  CHECK_I32(seq_start);
+  CHECK_I32(seq_slot);
+  CHECK_I32(seq_init);
+  TORCH_CHECK(seq_start.numel() == seq_slot.numel() + 1 && seq_init.numel() == seq_slot.numel(), "sequence tables");
+  (void)slots;
+}
+
+void embed_scale(Tensor ids, Tensor table, double scale, Tensor hist) {
+  const c10::hip::OptionalHIPGuard g(dev_of(ids));
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == torch::kInt64 && ids.is_contiguous(), "ids: int64");
+  TORCH_CHECK(table.is_cuda() && act_ok(table) && table.dim() == 2 && table.is_contiguous(), "table");
+  CHECK_F32(hist);
+  const int T = ids.numel(), d = table.size(1);
+  TORCH_CHECK(hist.dim() == 3 && hist.size(0) >= 2 && hist.size(1) == T && hist.size(2) == d, "hist [S, T, d]");
+  sm_embed_scale(ids.data_ptr<int64_t>(), table.data_ptr(), (float)scale, hist.data_ptr<float>(),
+                 hist.data_ptr<float>() + (int64_t)T * d, T, d, is_f32(table), cur());
+}
+
+void zc_norm(Tensor x, Tensor w, double eps, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(x));
+  CHECK_F32(x);
+  TORCH_CHECK(x.dim() == 2 && act_ok(w) && w.is_cuda() && w.is_contiguous() && w.numel() == x.size(1), "weight");
+  CHECK_ACT(out, w);
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes(), "out");
+  sm_zc_norm(x.data_ptr<float>(), w.data_ptr(), (float)eps, out.data_ptr(), x.size(0), x.size(1), is_f32(w), cur());
+}
+
+void add_post_norm(Tensor y, Tensor wp, Tensor ls, Tensor x, double eps, c10::optional<Tensor> wn,
+                   c10::optional<Tensor> out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(x));
+  CHECK_F32(x);
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && y.sizes() == x.sizes() && y.stride(1) == 1 && act_ok(y) && y.is_cuda(),
+              "y [T, d]");
+  const int T = x.size(0), d = x.size(1);
+  CHECK_ACT(wp, y);
+  CHECK_ACT(ls, y);
+  TORCH_CHECK(wp.is_contiguous() && ls.is_contiguous() && wp.numel() == d && ls.numel() == d, "weights");
+  const void* wnp = nullptr;
+  void* op = nullptr;
+  if (wn.has_value()) {
+    TORCH_CHECK(out.has_value(), "next norm without output");
+    CHECK_ACT(*wn, y);
+    CHECK_ACT(*out, y);
+    TORCH_CHECK(wn->is_contiguous() && wn->numel() == d && out->is_contiguous() && out->sizes() == x.sizes(), "next");
+    wnp = wn->data_ptr();
+    op = out->data_ptr();
+  }
+  sm_add_post_norm(y.data_ptr(), y.stride(0), wp.data_ptr(), ls.data_ptr(), x.data_ptr<float>(), (float)eps, wnp, op, T,
+                   d, is_f32(y), cur());
+}
+
+void depth_avg_norm(Tensor hist, int64_t n, Tensor coef, int64_t dst, Tensor w, double eps, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(hist));
+  CHECK_F32(hist);
+  CHECK_F32(coef);
+  TORCH_CHECK(hist.dim() == 3 && n >= 1 && n <= hist.size(0) && dst >= n && dst < hist.size(0) && coef.numel() >= n,
+              "depth average: n terms, destination behind them");
+  const int T = hist.size(1), d = hist.size(2);
+  TORCH_CHECK(w.is_cuda() && act_ok(w) && w.is_contiguous() && w.numel() == d, "weight");
+  CHECK_ACT(out, w);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == d, "out");
+  sm_depth_avg_norm(hist.data_ptr<float>(), (int64_t)T * d, n, coef.data_ptr<float>(), dst, w.data_ptr(), (float)eps,
+                    out.data_ptr(), T, d, is_f32(w), cur());
+}
+
+void xielu(Tensor z, double ap, double aq, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(z));
+  TORCH_CHECK(z.is_cuda() && act_ok(z) && z.is_contiguous(), "z");
+  CHECK_ACT(out, z);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == z.numel(), "out");
+  sm_xielu(z.data_ptr(), (float)ap, (float)aq, out.data_ptr(), z.numel(), is_f32(z), cur());
+}
+
+void softcap(Tensor x, double cap) {
+  const c10::hip::OptionalHIPGuard g(dev_of(x));
+  CHECK_F32(x);
+  TORCH_CHECK(cap > 0, "cap");
+  sm_softcap(x.data_ptr<float>(), (float)cap, x.numel(), cur());
+}
+
+void latent_rope_cache(Tensor q, Tensor kv, Tensor norm_w, double eps, Tensor positions, Tensor cos_sin, int64_t H,
+                       int64_t dn, int64_t dr, int64_t rot_dims, int64_t R, Tensor slots, Tensor cache, Tensor q_abs) {
+  const c10::hip::OptionalHIPGuard g(dev_of(q));
+  TORCH_CHECK(q.is_cuda() && act_ok(q) && q.dim() == 2 && q.stride(1) == 1 && q.size(1) == H * (dn + dr), "q");
+  const int T = q.size(0);
+  CHECK_ACT(kv, q);
+  TORCH_CHECK(kv.dim() == 2 && kv.stride(1) == 1 && kv.size(0) == T && kv.size(1) == R + dr, "kv");
+  CHECK_ACT(norm_w, q);
+  TORCH_CHECK(norm_w.is_contiguous() && norm_w.numel() == R, "latent norm weight");
+  TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == torch::kInt64 && positions.is_contiguous() &&
+                  positions.numel() == T, "positions");
+  TORCH_CHECK(slots.is_cuda() && slots.scalar_type() == torch::kInt64 && slots.is_contiguous() && slots.numel() == T,
+              "slots");
+  CHECK_F32(cos_sin);
+  TORCH_CHECK(cos_sin.dim() == 2 && cos_sin.size(1) == rot_dims && rot_dims % 2 == 0 && rot_dims <= dr, "rotary table");
+  CHECK_ACT(cache, q);
+  TORCH_CHECK(cache.dim() == 3 && cache.is_contiguous() && cache.size(2) == R + dr, "cache [blocks, bs, R + dr]");
+  CHECK_ACT(q_abs, q);
+  TORCH_CHECK(q_abs.is_contiguous() && q_abs.numel() == (int64_t)T * H * (R + dr), "q_abs");
+  // positions and slots are produced by the runner within [0, max_pos) and the pool
+  sm_latent_rope_cache(q.data_ptr(), q.stride(0), kv.data_ptr(), kv.stride(0), norm_w.data_ptr(), (float)eps,
+                       positions.data_ptr<int64_t>(), cos_sin.data_ptr<float>(), H, dn, dr, rot_dims, R,
+                       slots.data_ptr<int64_t>(), cache.data_ptr(), q_abs.data_ptr(), T, is_f32(q), cur());
+}
+
+void latent_attention(Tensor q_abs, Tensor cache, Tensor tables, Tensor row_seq, Tensor row_len, double scale,
+                      int64_t R, int64_t qt, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(q_abs));
+  TORCH_CHECK(q_abs.is_cuda() && act_ok(q_abs) && q_abs.dim() == 3 && q_abs.is_contiguous(), "q_abs [T, H, Dk]");
+  const int T = q_abs.size(0), H = q_abs.size(1), Dk = q_abs.size(2);
+  CHECK_ACT(cache, q_abs);
+  TORCH_CHECK(cache.dim() == 3 && cache.is_contiguous() && cache.size(2) == Dk && R >= 1 && R <= Dk, "cache");
+  CHECK_I32(tables);
+  CHECK_I32(row_seq);
+  CHECK_I32(row_len);
+  TORCH_CHECK(tables.dim() == 2 && row_seq.numel() == T && row_len.numel() == T, "row tables");
+  CHECK_ACT(out, q_abs);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == (int64_t)T * H * R, "out [T, H, R]");
+  TORCH_CHECK(qt == 1 || qt == 4, "rows per workgroup: 1 or 4");
+  const int rc = sm_latent_attention(q_abs.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
+                                     cache.size(1), row_seq.data_ptr<int>(), row_len.data_ptr<int>(), (float)scale, H,
+                                     R, Dk, T, qt, out.data_ptr(), is_f32(q_abs), cur());
+  TORCH_CHECK(rc == 0, "latent_attention: latent rank above 1024 or rows too wide for the LDS tile");
+}
+
+void causal_conv_silu(Tensor xz, int64_t C, Tensor w, Tensor b, Tensor state, Tensor seq_start, Tensor seq_slot,
+                      Tensor seq_init, int64_t max_q, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(xz));
+  TORCH_CHECK(xz.is_cuda() && act_ok(xz) && xz.dim() == 2 && xz.stride(1) == 1 && xz.size(1) >= C, "xz");
+  CHECK_ACT(w, xz);
+  CHECK_ACT(b, xz);
+  CHECK_ACT(state, xz);
+  CHECK_ACT(out, xz);
+  TORCH_CHECK(w.dim() == 2 && w.is_contiguous() && w.size(0) == C && b.is_contiguous() && b.numel() == C, "conv weights");
+  const int taps = w.size(1);
+  TORCH_CHECK(state.dim() == 3 && state.is_contiguous() && state.size(2) == C && state.size(1) >= taps - 1 &&
+                  (taps == 1 || state.size(1) == taps - 1), "conv state [slots, taps-1, C]");
+  check_seq(seq_start, seq_slot, seq_init, state.size(0));
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == xz.size(0) && out.size(1) == C, "out");
+  sm_causal_conv_silu(xz.data_ptr(), xz.stride(0), C, w.data_ptr(), b.data_ptr(), taps, state.data_ptr(),
+                      seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(), out.data_ptr(),
+                      seq_slot.numel(), max_q, is_f32(xz), cur());
+}
+
+void selective_scan(Tensor xc, Tensor dt_raw, Tensor dt_bias, Tensor A, Tensor bc, int64_t R, int64_t N, Tensor D,
+                    Tensor xz, int64_t C, Tensor state, Tensor seq_start, Tensor seq_slot, Tensor seq_init, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(xc));
+  TORCH_CHECK(xc.is_cuda() && act_ok(xc) && xc.dim() == 2 && xc.is_contiguous() && xc.size(1) == C, "xc");
+  const int T = xc.size(0);
+  CHECK_ACT(dt_raw, xc);
+  CHECK_ACT(dt_bias, xc);
+  CHECK_ACT(bc, xc);
+  CHECK_ACT(D, xc);
+  CHECK_ACT(xz, xc);
+  CHECK_ACT(out, xc);
+  CHECK_F32(A);
+  CHECK_F32(state);
+  TORCH_CHECK(dt_raw.is_contiguous() && dt_raw.sizes() == xc.sizes() && dt_bias.numel() == C && D.numel() == C &&
+                  dt_bias.is_contiguous() && D.is_contiguous(), "dt / D");
+  TORCH_CHECK(A.dim() == 2 && A.size(0) == C && A.size(1) == N, "A [C, N]");
+  TORCH_CHECK(bc.dim() == 2 && bc.stride(1) == 1 && bc.size(0) == T && bc.size(1) >= R + 2 * N, "bc");
+  TORCH_CHECK(xz.dim() == 2 && xz.stride(1) == 1 && xz.size(0) == T && xz.size(1) >= 2 * C, "xz");
+  TORCH_CHECK(state.dim() == 3 && state.size(1) == C && state.size(2) == N, "state [slots, C, N]");
+  check_seq(seq_start, seq_slot, seq_init, state.size(0));
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == xc.sizes(), "out");
+  const int rc = sm_selective_scan(xc.data_ptr(), dt_raw.data_ptr(), dt_bias.data_ptr(), A.data_ptr<float>(),
+                                   bc.data_ptr(), bc.stride(0), R, N, D.data_ptr(), xz.data_ptr(), xz.stride(0), C,
+                                   state.data_ptr<float>(), seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(),
+                                   seq_init.data_ptr<int>(), out.data_ptr(), seq_slot.numel(), is_f32(xc), cur());
+  TORCH_CHECK(rc == 0, "selective_scan: state size above 256");
+}
+
+void gdelta_scan(Tensor proj, Tensor wl, Tensor w0, Tensor a_b, Tensor norm_w, double eps, int64_t H, int64_t d,
+                 Tensor state, Tensor seq_start, Tensor seq_slot, Tensor seq_init, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(proj));
+  const int64_t HD = H * d;
+  TORCH_CHECK(proj.is_cuda() && act_ok(proj) && proj.dim() == 2 && proj.stride(1) == 1 && proj.size(1) >= 5 * HD, "proj");
+  const int T = proj.size(0);
+  CHECK_ACT(wl, proj);
+  CHECK_ACT(w0, proj);
+  CHECK_ACT(a_b, proj);
+  CHECK_ACT(norm_w, proj);
+  CHECK_ACT(out, proj);
+  CHECK_F32(state);
+  TORCH_CHECK(wl.is_contiguous() && wl.dim() == 2 && wl.size(0) == T && wl.size(1) == HD, "decay logits");
+  TORCH_CHECK(w0.is_contiguous() && a_b.is_contiguous() && norm_w.is_contiguous() && w0.numel() == HD &&
+                  a_b.numel() == HD && norm_w.numel() == HD, "per-channel vectors");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == d && state.size(3) == d, "state");
+  check_seq(seq_start, seq_slot, seq_init, state.size(0));
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == HD, "out");
+  const int rc = sm_gdelta_scan(proj.data_ptr(), proj.stride(0), wl.data_ptr(), w0.data_ptr(), a_b.data_ptr(),
+                                norm_w.data_ptr(), (float)eps, H, d, state.data_ptr<float>(),
+                                seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(),
+                                out.data_ptr(), seq_slot.numel(), is_f32(proj), cur());
+  TORCH_CHECK(rc == 0, "gdelta_scan: head size above 256");
+}
+
+void moe_route(Tensor logits, int64_t k, Tensor ids, Tensor w) {
+  const c10::hip::OptionalHIPGuard g(dev_of(logits));
+  CHECK_F32(logits);
+  CHECK_I32(ids);
+  CHECK_F32(w);
+  const int T = logits.size(0), E = logits.size(1);
+  TORCH_CHECK(logits.dim() == 2 && k >= 1 && k <= E && ids.numel() == (int64_t)T * k && w.numel() == (int64_t)T * k,
+              "router shapes");
+  sm_moe_route(logits.data_ptr<float>(), E, k, ids.data_ptr<int>(), w.data_ptr<float>(), T, cur());
+}
+
+void moe_group(Tensor ids, int64_t E, Tensor slot_row, Tensor tile_e, Tensor pair_slot) {
+  const c10::hip::OptionalHIPGuard g(dev_of(ids));
+  CHECK_I32(ids);
+  CHECK_I32(slot_row);
+  CHECK_I32(tile_e);
+  CHECK_I32(pair_slot);
+  const int64_t n = ids.numel(), mt = tile_e.numel();
+  TORCH_CHECK(slot_row.numel() == mt * 64 && pair_slot.numel() == n && mt * 64 >= n + E * 63 && E <= 8192,
+              "tile tables too small for n pairs over E experts");
+  sm_moe_group(ids.data_ptr<int>(), n, E, slot_row.data_ptr<int>(), tile_e.data_ptr<int>(), pair_slot.data_ptr<int>(),
+               mt, cur());
+}
+
+void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, Tensor C, bool gelu) {
+  const c10::hip::OptionalHIPGuard g(dev_of(A));
+  TORCH_CHECK(A.is_cuda() && act_ok(A) && A.dim() == 2 && A.stride(1) == 1, "A");
+  CHECK_ACT(W, A);
+  CHECK_ACT(C, A);
+  CHECK_I32(slot_row);
+  CHECK_I32(tile_e);
+  TORCH_CHECK(W.dim() == 3 && W.is_contiguous() && W.size(2) == A.size(1), "W [E, N, K]");
+  const int64_t mt = tile_e.numel();
+  TORCH_CHECK(slot_row.numel() == mt * 64 && C.is_contiguous() && C.dim() == 2 && C.size(0) == mt * 64 &&
+                  C.size(1) == W.size(1), "C [tiles * 64, N]");
+  TORCH_CHECK(kdiv > 0 || A.size(0) == mt * 64, "A rows are the tile slots");
+  sm_moe_gemm(A.data_ptr(), A.stride(0), kdiv, slot_row.data_ptr<int>(), tile_e.data_ptr<int>(), W.data_ptr(),
+              W.size(1), W.size(2), C.data_ptr(), mt, gelu ? 1 : 0, is_f32(A), cur());
+}
+
+void moe_combine(Tensor y, Tensor pair_slot, Tensor w, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(y));
+  TORCH_CHECK(y.is_cuda() && act_ok(y) && y.dim() == 2 && y.is_contiguous(), "y");
+  CHECK_I32(pair_slot);
+  CHECK_F32(w);
+  CHECK_ACT(out, y);
+  const int T = out.size(0), d = out.size(1);
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && y.size(1) == d && w.dim() == 2 && w.size(0) == T &&
+                  pair_slot.numel() == w.numel(), "combine shapes");
+  sm_moe_combine(y.data_ptr(), pair_slot.data_ptr<int>(), w.data_ptr<float>(), w.size(1), d, out.data_ptr(), T,
+                 is_f32(y), cur());
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("embed_scale", &embed_scale);
+  m.def("zc_norm", &zc_norm);
+  m.def("add_post_norm", &add_post_norm);
+  m.def("depth_avg_norm", &depth_avg_norm);
+  m.def("xielu", &xielu);
+  m.def("softcap", &softcap);
+  m.def("latent_rope_cache", &latent_rope_cache);
+  m.def("latent_attention", &latent_attention);
+  m.def("causal_conv_silu", &causal_conv_silu);
+  m.def("selective_scan", &selective_scan);
+  m.def("gdelta_scan", &gdelta_scan);
+  m.def("moe_route", &moe_route);
+  m.def("moe_group", &moe_group);
+  m.def("moe_gemm", &moe_gemm);
+  m.def("moe_combine", &moe_combine);
+}

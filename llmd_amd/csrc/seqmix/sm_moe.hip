@@ -1,0 +1,197 @@
+// Ungated mixture-of-experts feed-forward: W_down gelu(W_up h) per chosen expert.
+//
+// moe_route   : top-k of fp32 router logits (ties to the lower index), softmax over the chosen.
+// moe_group   : one workgroup sorts the (token, choice) pairs by expert into 64-row tiles
+//               (counts and ranks through LDS atomics; a tile holds rows of one expert only).
+// moe_gemm    : tile GEMM, 64 rows x 64 columns per workgroup, K stepped by 16 through LDS,
+//               4 x 4 outputs per thread, fp32 accumulation in a fixed K order (a row's sums do
+//               not depend on its tile or on the rest of the step); optional erf-GELU epilogue.
+// moe_combine : out[t] = sum_j w[t, j] * y[slot(t, j)] in fp32.
+#include "seqmix_common.h"
+
+using namespace sm;
+
+namespace {
+
+constexpr int TM = 64, TN = 64, TK = 16;
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int E, int k,
+                                                        int* __restrict__ ids, float* __restrict__ w, int T) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + (int64_t)t * E;
+  int* oi = ids + (int64_t)t * k;
+  float* ow = w + (int64_t)t * k;
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY;
+    int bi = -1;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int i = 0; i < j; ++i) taken |= oi[i] == e;
+      const float v = z[e];
+      if (!taken && (bi < 0 || v > best)) {
+        best = v;
+        bi = e;
+      }
+    }
+    oi[j] = bi;
+    ow[j] = best;
+  }
+  const float m = ow[0];  // the first chosen is the largest
+  float s = 0.f;
+  for (int j = 0; j < k; ++j) {
+    const float p = expf(ow[j] - m);
+    ow[j] = p;
+    s += p;
+  }
+  for (int j = 0; j < k; ++j) ow[j] /= s;
+}
+
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int n, int E,
+                                                         int* __restrict__ slot_row, int* __restrict__ tile_e,
+                                                         int* __restrict__ pair_slot, int max_tiles) {
+  extern __shared__ int sh[];  // cnt[E] | first_tile[E]
+  int* cnt = sh;
+  int* first = sh + E;
+  for (int e = threadIdx.x; e < E; e += 1024) cnt[e] = 0;
+  for (int i = threadIdx.x; i < max_tiles * TM; i += 1024) slot_row[i] = -1;
+  for (int i = threadIdx.x; i < max_tiles; i += 1024) tile_e[i] = -1;
+  __syncthreads();
+  for (int p = threadIdx.x; p < n; p += 1024) atomicAdd(&cnt[ids[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int tile = 0;
+    for (int e = 0; e < E; ++e) {
+      first[e] = tile;
+      const int nt = (cnt[e] + TM - 1) / TM;
+      for (int i = 0; i < nt; ++i) tile_e[tile + i] = e;
+      tile += nt;
+      cnt[e] = 0;  // reused as the running rank
+    }
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < n; p += 1024) {
+    const int e = ids[p];
+    const int slot = first[e] * TM + atomicAdd(&cnt[e], 1);
+    slot_row[slot] = p;
+    pair_slot[p] = slot;
+  }
+}
+
+// C[slot, n] = act(sum_k A[row(slot), k] * W[e, n, k]);  row(slot) = pair / kdiv (gathered
+// tokens) when kdiv > 0, the slot itself otherwise.
+template <typename T, bool GELU>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, int64_t a_stride, int kdiv,
+                                                       const int* __restrict__ slot_row,
+                                                       const int* __restrict__ tile_e, const T* __restrict__ Wt,
+                                                       int N, int K, T* __restrict__ Cout) {
+  const int e = tile_e[blockIdx.x];
+  if (e < 0) return;
+  __shared__ float sA[TK][TM + 4], sB[TK][TN + 4];
+  __shared__ int srow[TM];
+  const int tid = threadIdx.x;
+  const int slot0 = blockIdx.x * TM, n0 = blockIdx.y * TN;
+  if (tid < TM) {
+    const int p = slot_row[slot0 + tid];
+    srow[tid] = p < 0 ? -1 : (kdiv > 0 ? p / kdiv : slot0 + tid);
+  }
+  __syncthreads();
+  const T* We = Wt + (int64_t)e * N * K;
+  const int lr = tid >> 2, lk = (tid & 3) * 4;  // loader: row / column lr, 4 consecutive k
+  const int ty = tid >> 4, tx = tid & 15;       // compute: rows ty*4.., columns tx*4..
+  float acc[4][4] = {};
+  const int arow = srow[lr];
+  const int brow = n0 + lr;
+  for (int k0 = 0; k0 < K; k0 += TK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int kk = k0 + lk + i;
+      sA[lk + i][lr] = (arow >= 0 && kk < K) ? ld(A + (int64_t)arow * a_stride + kk) : 0.f;
+      sB[lk + i][lr] = (brow < N && kk < K) ? ld(We + (int64_t)brow * K + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < TK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[i] = sA[kk][ty * 4 + i];
+        b[i] = sB[kk][tx * 4 + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * b[j];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ty * 4 + i;
+    if (srow[r] < 0) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= N) continue;
+      float v = acc[i][j];
+      if (GELU) v = 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
+      st(Cout + (int64_t)(slot0 + r) * N + n, v);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ pair_slot,
+                                                          const float* __restrict__ w, int k, int d,
+                                                          T* __restrict__ out) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    float s = 0.f;
+    for (int j = 0; j < k; ++j) s += w[t * k + j] * ld(y + (int64_t)pair_slot[t * k + j] * d + c);
+    st(out + t * d + c, s);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+void sm_moe_route(const float* logits, int E, int k, int* ids, float* w, int T, hipStream_t stream) {
+  if (T == 0) return;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, stream, logits, E, k, ids, w, T);
+}
+
+void sm_moe_group(const int* ids, int n, int E, int* slot_row, int* tile_e, int* pair_slot, int max_tiles,
+                  hipStream_t stream) {
+  hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 2 * E * sizeof(int), stream, ids, n, E, slot_row, tile_e,
+                     pair_slot, max_tiles);
+}
+
+void sm_moe_gemm(const void* A, int64_t a_stride, int kdiv, const int* slot_row, const int* tile_e, const void* W,
+                 int N, int K, void* C, int max_tiles, int gelu, int f32, hipStream_t stream) {
+  const dim3 grid(max_tiles, (N + TN - 1) / TN);
+#define SM_GO(TYPE, G)                                                                                          \
+  hipLaunchKernelGGL((moe_gemm_kernel<TYPE, G>), grid, dim3(256), 0, stream, (const TYPE*)A, a_stride, kdiv,   \
+                     slot_row, tile_e, (const TYPE*)W, N, K, (TYPE*)C)
+  if (f32) {
+    if (gelu) SM_GO(float, true);
+    else SM_GO(float, false);
+  } else {
+    if (gelu) SM_GO(bf16_t, true);
+    else SM_GO(bf16_t, false);
+  }
+#undef SM_GO
+}
+
+void sm_moe_combine(const void* y, const int* pair_slot, const float* w, int k, int d, void* out, int T, int f32,
+                    hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    hipLaunchKernelGGL((moe_combine_kernel<float>), dim3(T), dim3(256), 0, stream, (const float*)y, pair_slot, w, k, d,
+                       (float*)out);
+  else
+    hipLaunchKernelGGL((moe_combine_kernel<bf16_t>), dim3(T), dim3(256), 0, stream, (const bf16_t*)y, pair_slot, w, k,
+                       d, (bf16_t*)out);
+}
+
+}  // extern "C"

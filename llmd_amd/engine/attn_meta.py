@@ -25,7 +25,8 @@ class SeqMeta:
     row_seq: torch.Tensor            # [T] int32: token -> sequence (row of ``tables``)
     row_len: torch.Tensor            # [T] int32: keys the token sees (= position + 1)
     tables: torch.Tensor             # [n, W] int32 block tables
-    max_len: int = 0
+    max_len: int = 0                 # longest context of the step
+    max_q: int = 0                   # longest run of the step
 
 
 @dataclass

@@ -135,7 +135,7 @@ class MekusunForCausalLM(torch.nn.Module):
 
     @torch.no_grad()
     def compute_logits(self, h):
-        logits = self.lm_head(h).float()
+        logits = self.lm_head(h).float().contiguous()
         if self.cfg.logit_softcap:
             sm.softcap_(logits, self.cfg.logit_softcap)
         return logits

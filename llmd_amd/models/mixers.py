@@ -84,7 +84,8 @@ class LatentAttention(torch.nn.Module):
         # absorb W_uk into the query: scores against the latent itself
         qn = q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1)                       # [H, T, dn]
         q_abs[:, :, :R].copy_(torch.bmm(qn, self.uk.view(H, dn, R)).transpose(0, 1))
-        o_lat = sm.latent_attention(q_abs, self.cache, s.tables, s.row_seq, s.row_len, self.scale, R)
+        o_lat = sm.latent_attention(q_abs, self.cache, s.tables, s.row_seq, s.row_len, self.scale, R,
+                                    rows_per_group=4 if s.max_q > 1 else 1)
         o = torch.bmm(o_lat.transpose(0, 1), self.uv.view(H, self.dv, R).transpose(1, 2))  # [H, T, dv]
         return self.o(o.transpose(0, 1).reshape(T, H * self.dv))
 
@@ -120,7 +121,7 @@ class Mamba1Mixer(torch.nn.Module):
         s = meta.seq
         xz = self.in_proj(h)
         xc = sm.causal_conv_silu(xz, self.C, self.conv, self.conv_b, self.conv_state, s.seq_start, s.seq_slot,
-                                 s.seq_init)
+                                 s.seq_init, s.max_q)
         bc = self.x_proj(xc)
         dt_raw = self.dt_proj(bc[:, :self.R])
         y = sm.selective_scan(xc, dt_raw, self.dt_b, self.A, bc, self.R, self.N, self.D, xz, self.C,

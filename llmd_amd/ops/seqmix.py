@@ -84,25 +84,27 @@ def latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dim
                                q_abs)
 
 
-def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: int, max_len: int = 0):
+def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: int, rows_per_group: int = 1):
     """Causal softmax attention of absorbed queries [T, H, R + dr] over the paged latent cache
     [blocks, bs, R + dr]; row t sees the first row_len[t] keys of sequence row_seq[t].
-    Returns the latent outputs [T, H, R]."""
+    Returns the latent outputs [T, H, R]. ``rows_per_group`` (1 or 4): consecutive rows that share
+    a workgroup's key tiles - 4 for steps with prompt portions, 1 for decode-only steps."""
     T, H, _ = q_abs.shape
     out = torch.empty(T, H, R, dtype=q_abs.dtype, device=q_abs.device)
     if not q_abs.is_cuda:
         return ref.latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out)
-    native().latent_attention(q_abs, cache, tables, row_seq, row_len, float(scale), R, out)
+    native().latent_attention(q_abs, cache, tables, row_seq, row_len, float(scale), R, int(rows_per_group), out)
     return out
 
 
-def causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init):
+def causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init, max_q: int):
     """Per-channel causal convolution + SiLU over the first C columns of xz, continuing from each
-    sequence's last taps-1 inputs in ``conv_state`` [slots, taps-1, C] (updated)."""
+    sequence's last taps-1 inputs in ``conv_state`` [slots, taps-1, C] (updated). ``max_q``: the
+    longest run of the step (sizes the grid)."""
     out = torch.empty(xz.shape[0], C, dtype=xz.dtype, device=xz.device)
     if not xz.is_cuda:
         return ref.causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init, out)
-    native().causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init, out)
+    native().causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init, int(max_q), out)
     return out
 
 
