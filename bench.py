@@ -90,6 +90,11 @@ def _reference(model: str, value: float, n_gpus: int) -> dict:
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--mixer-bench", action="store_true",
+                   help="instead of the serving workload: prefill / decode throughput of the per-layer stacks "
+                        "(latent attention + experts, selective scan, delta rule) at model-like sizes beside "
+                        "DeepSeek-V2-Lite layers of equal size (llmd_amd/tools/mixer_bench.py; uses --isl as "
+                        "the context and --concurrency as the decode batch when they are given)")
     p.add_argument("--steps", type=int, default=40)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--model", default="llama-3-70b")
@@ -149,6 +154,12 @@ def log(rank, *a):
 
 def main():
     a = parse()
+    if a.mixer_bench:  # a different workload; the default one and its output line are unchanged
+        from llmd_amd.tools import mixer_bench
+
+        ctx = a.isl if a.isl != 5000 else 2048
+        print(json.dumps(mixer_bench.run(tokens=ctx, batch=min(a.concurrency, 64))), flush=True)
+        return
     if os.environ.get("LLMD_BENCH_STACKS"):
         import faulthandler
 

@@ -8,7 +8,7 @@
 #include <hip/hip_runtime.h>
 
 extern "C" {
-void sm_embed_scale(const int64_t*, const void*, float, float*, float*, int, int, int, hipStream_t);
+void sm_embed_scale(const int64_t*, const void*, float, float*, float*, int, int, int64_t, int, hipStream_t);
 void sm_zc_norm(const float*, const void*, float, void*, int, int, int, hipStream_t);
 void sm_add_post_norm(const void*, int64_t, const void*, const void*, float*, float, const void*, void*, int, int, int,
                       hipStream_t);
@@ -68,7 +68,7 @@ void embed_scale(Tensor ids, Tensor table, double scale, Tensor hist) {
   const int T = ids.numel(), d = table.size(1);
   TORCH_CHECK(hist.dim() == 3 && hist.size(0) >= 2 && hist.size(1) == T && hist.size(2) == d, "hist [S, T, d]");
   sm_embed_scale(ids.data_ptr<int64_t>(), table.data_ptr(), (float)scale, hist.data_ptr<float>(),
-                 hist.data_ptr<float>() + (int64_t)T * d, T, d, is_f32(table), cur());
+                 hist.data_ptr<float>() + (int64_t)T * d, T, d, table.size(0), is_f32(table), cur());
 }
 
 void zc_norm(Tensor x, Tensor w, double eps, Tensor out) {

@@ -13,9 +13,10 @@ constexpr int NT = 256;
 template <typename T>
 __global__ __launch_bounds__(NT) void embed_scale_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table,
                                                         float scale, float* __restrict__ o0, float* __restrict__ o1,
-                                                        int d) {
+                                                        int d, int64_t V) {
   const int64_t row = blockIdx.x;
-  const T* src = table + ids[row] * (int64_t)d;
+  const int64_t id = min(max(ids[row], (int64_t)0), V - 1);  // a bad id must not read outside the table
+  const T* src = table + id * (int64_t)d;
   for (int c = threadIdx.x; c < d; c += NT) {
     const float v = ld(src + c) * scale;
     o0[row * d + c] = v;
@@ -110,11 +111,11 @@ __global__ __launch_bounds__(NT) void softcap_kernel(float* __restrict__ x, floa
 
 extern "C" {
 
-void sm_embed_scale(const int64_t* ids, const void* table, float scale, float* o0, float* o1, int T, int d, int f32,
-                    hipStream_t stream) {
+void sm_embed_scale(const int64_t* ids, const void* table, float scale, float* o0, float* o1, int T, int d,
+                    int64_t V, int f32, hipStream_t stream) {
   if (T == 0) return;
-  if (f32) hipLaunchKernelGGL((embed_scale_kernel<float>), dim3(T), dim3(NT), 0, stream, ids, (const float*)table, scale, o0, o1, d);
-  else hipLaunchKernelGGL((embed_scale_kernel<bf16_t>), dim3(T), dim3(NT), 0, stream, ids, (const bf16_t*)table, scale, o0, o1, d);
+  if (f32) hipLaunchKernelGGL((embed_scale_kernel<float>), dim3(T), dim3(NT), 0, stream, ids, (const float*)table, scale, o0, o1, d, V);
+  else hipLaunchKernelGGL((embed_scale_kernel<bf16_t>), dim3(T), dim3(NT), 0, stream, ids, (const bf16_t*)table, scale, o0, o1, d, V);
 }
 
 void sm_zc_norm(const float* x, const void* w, float eps, void* out, int T, int d, int f32, hipStream_t stream) {

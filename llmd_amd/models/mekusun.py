@@ -135,10 +135,11 @@ class MekusunForCausalLM(torch.nn.Module):
 
     @torch.no_grad()
     def compute_logits(self, h):
-        logits = self.lm_head(h).float().contiguous()
+        # over the head's padded rows, so that the rows stay 16-byte aligned for the sampling kernel
+        logits = torch.nn.functional.linear(h, self.lm_head.weight).float()
         if self.cfg.logit_softcap:
             sm.softcap_(logits, self.cfg.logit_softcap)
-        return logits
+        return logits[:, :self.cfg.vocab_size]
 
     def weight_specs(self) -> list:
         specs = [("embed", self.embed.weight, "vocab", None), ("final.norm", self.norm, "replicate", None),

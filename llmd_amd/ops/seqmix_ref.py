@@ -77,7 +77,7 @@ def causal_conv_silu(xz, C, w, b, conv_state, seq_start, seq_slot, seq_init, out
     for i in range(seq_slot.numel()):
         lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
         x = xz[lo:hi, :C].float()
-        prev = conv_state[sl].float() if int(seq_init[i]) else torch.zeros(taps - 1, C)
+        prev = conv_state[sl, :taps - 1].float() if int(seq_init[i]) else torch.zeros(taps - 1, C)
         xp = torch.cat([prev, x])
         acc = bf.expand(hi - lo, C).clone()
         for j in range(taps):

@@ -1,0 +1,133 @@
+"""Prefill and decode throughput of per-layer stacks at sizes that resemble a real model's
+layers (random weights), beside the closest existing model at equal size.
+
+``python bench.py --mixer-bench`` runs it; the default bench workload is unchanged. Three
+Mekusun stacks of DeepSeek-V2-Lite's width (2048) are timed through the runner's own step
+(``ModelRunner.run_plan``: the kernels, cache writes and state updates of serving):
+
+  latent+moe : latent attention 16 heads x (128 + 64), value 128, latent 512; 64 experts, 6 chosen,
+               ff 1408 - the geometry of DeepSeek-V2-Lite's layers, which run beside it
+               (models/deepseek.py: MLA kernels of fixed size, gated experts + shared expert)
+  mamba      : selective scan, inner 4096, state 16, dt rank 128, 4 taps; dense ff 5632
+  delta      : generalized delta rule, 32 heads x 64; dense ff 5632
+
+Prefill: one prompt of ``--tokens`` tokens in one step. Decode: ``--batch`` sequences with that
+context, one token each. One JSON line with tokens/s and ms per layer for every entry.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import time
+
+import numpy as np
+import torch
+
+WIDTH = 2048
+
+
+def _attn():
+    return {"type": "latent_attention",
+            "mixer": {"heads": 16, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+                      "rot": {"dims": 64, "base": 10000.0}},
+            "mlp": {"kind": "moe", "expert": {"ff": 1408}, "router": {"experts": 64, "top": 6}}}
+
+
+def _mamba():
+    return {"type": "mamba1", "mixer": {"inner": 4096, "state": 16, "dt_rank": 128, "conv": 4},
+            "mlp": {"kind": "dense", "ff": 5632}}
+
+
+def _delta():
+    return {"type": "general_delta", "mixer": {"heads": 32, "dim": 64, "decay_rank": 64},
+            "mlp": {"kind": "dense", "ff": 5632}}
+
+
+def stack_config(layer: dict, n_layers: int):
+    from llmd_amd.engine.config import mekusun_config
+
+    return mekusun_config({"architecture": "Mekusun", "width": WIDTH, "vocab": 32000, "embedding": {"scale": 1.0},
+                           "logit_softcap": 30.0, "norm": {"eps": 1e-6}, "layers": [layer] * n_layers})
+
+
+def _runner(mc, tokens: int, batch: int, device: str):
+    from llmd_amd.engine.config import EngineConfig
+    from llmd_amd.engine.model_runner import ModelRunner
+
+    bs = 64
+    pages = (batch + 1) * (tokens // bs + 2)
+    cfg = EngineConfig.create(mc.name, model_config=mc, device=device, block_size=bs, num_gpu_blocks=pages,
+                              max_num_seqs=batch + 1, max_model_len=tokens + 65, max_num_batched_tokens=tokens,
+                              enforce_eager=True, enable_prefix_caching=False, prefill_token_align=0)
+    r = ModelRunner(cfg)
+    r.profile_and_allocate()
+    return r
+
+
+def _plans(r, tokens: int, batch: int):
+    bs, W = r.bs, r.width
+    nb = tokens // bs + 2
+    rng = np.random.default_rng(0)
+    p_bt = np.zeros((1, W), np.int32)
+    p_bt[0, :nb] = np.arange(nb)
+    pre = {"graph": False, "nd": 0, "ids": rng.integers(0, 1000, tokens).tolist(), "pos": list(range(tokens)),
+           "slots": list(range(tokens)), "d_bt": np.zeros((0, W), np.int32), "d_len": np.zeros(0, np.int32),
+           "p_ql": [tokens], "p_ctx": [tokens], "p_bt": p_bt, "rows": [tokens - 1]}
+    d_bt = np.zeros((batch, W), np.int32)
+    for b in range(batch):
+        d_bt[b, :nb] = np.arange(nb) + (b + 1) * nb
+    dec = {"graph": False, "nd": batch, "ids": rng.integers(0, 1000, batch).tolist(), "pos": [tokens] * batch,
+           "slots": [int(d_bt[b, tokens // bs]) * bs + tokens % bs for b in range(batch)], "d_bt": d_bt,
+           "d_len": np.full(batch, tokens + 1, np.int32), "p_ql": [], "p_ctx": [],
+           "p_bt": np.zeros((0, W), np.int32), "rows": list(range(batch))}
+    if r.stateful:
+        pre["seq"] = ([0], [0])
+        dec["seq"] = (list(range(1, batch + 1)), [1] * batch)
+    return pre, dec
+
+
+def _time(r, pl, reps: int) -> float:
+    for _ in range(2):
+        r.run_plan(pl)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        r.run_plan(pl)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps
+
+
+def run(tokens: int = 2048, batch: int = 32, n_layers: int = 4, reps: int = 5, device: str = "cuda") -> dict:
+    import dataclasses
+
+    from llmd_amd.engine.config import get_model_config
+
+    out = {"tokens": tokens, "batch": batch, "layers": n_layers, "dtype": "bf16", "data": "synthetic", "entries": {}}
+    ref = dataclasses.replace(get_model_config("deepseek-v2-lite"), num_hidden_layers=n_layers + 1,
+                              first_k_dense_replace=1, vocab_size=32000, rope_scaling=None, name="deepseek-v2-lite-cut")
+    todo = [("latent+moe", stack_config(_attn(), n_layers), n_layers), ("mamba", stack_config(_mamba(), n_layers), n_layers),
+            ("delta", stack_config(_delta(), n_layers), n_layers), ("deepseek-v2-lite (1 dense + moe layers)", ref, n_layers + 1)]
+    for name, mc, L in todo:
+        r = _runner(mc, tokens, batch, device)
+        pre, dec = _plans(r, tokens, batch)
+        tp, td = _time(r, pre, reps), _time(r, dec, reps * 4)
+        out["entries"][name] = {"prefill_tok_s": round(tokens / tp), "prefill_ms_per_layer": round(tp * 1e3 / L, 3),
+                                "decode_tok_s": round(batch / td), "decode_ms_per_layer": round(td * 1e3 / L, 3)}
+        del r
+        torch.cuda.empty_cache()
+    return out
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--tokens", type=int, default=2048)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--layers", type=int, default=4)
+    ap.add_argument("--reps", type=int, default=5)
+    a = ap.parse_args(argv)
+    print(json.dumps(run(a.tokens, a.batch, a.layers, a.reps)), flush=True)
+
+
+if __name__ == "__main__":
+    main()
