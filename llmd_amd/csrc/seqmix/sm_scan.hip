@@ -89,24 +89,42 @@ __global__ __launch_bounds__(NT) void selective_scan_kernel(
     S[i] = (n < N && seq_init[s]) ? sp[n] : 0.f;
   }
   const float bias = ld(dt_bias + cc), Dc = ld(D + cc);
-  for (int t = lo; t < hi; ++t) {
-    const float dt = softplusf_(ld(dt_raw + (int64_t)t * C + cc) + bias);
-    const float x = ld(xc + (int64_t)t * C + cc);
+  // inputs are fetched one token ahead of the recurrence
+  float ndt = 0.f, nx = 0.f, nz = 0.f, nB[SPL], nC[SPL];
+  auto fetch = [&](int t) {
+    if (t >= hi) return;
+    ndt = ld(dt_raw + (int64_t)t * C + cc);
+    nx = ld(xc + (int64_t)t * C + cc);
+    nz = ld(xz + (int64_t)t * xz_stride + C + cc);
     const T* bt = bc + (int64_t)t * bc_stride + R;
+#pragma unroll
+    for (int i = 0; i < SPL; ++i) {
+      const int n = nl + i * NL;
+      nB[i] = n < N ? ld(bt + n) : 0.f;
+      nC[i] = n < N ? ld(bt + N + n) : 0.f;
+    }
+  };
+  fetch(lo);
+  for (int t = lo; t < hi; ++t) {
+    const float dt = softplusf_(ndt + bias), x = nx, z = nz;
+    float Bv[SPL], Cv[SPL];
+#pragma unroll
+    for (int i = 0; i < SPL; ++i) {
+      Bv[i] = nB[i];
+      Cv[i] = nC[i];
+    }
+    fetch(t + 1);
     float part = 0.f;
 #pragma unroll
     for (int i = 0; i < SPL; ++i) {
       const int n = nl + i * NL;
       if (n < N) {
-        S[i] = expf(dt * Ac[i]) * S[i] + dt * x * ld(bt + n);
-        part += S[i] * ld(bt + N + n);
+        S[i] = expf(dt * Ac[i]) * S[i] + dt * x * Bv[i];
+        part += S[i] * Cv[i];
       }
     }
     for (int o = NL >> 1; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
-    if (ok && nl == 0) {
-      const float z = ld(xz + (int64_t)t * xz_stride + C + c);
-      st(out + (int64_t)t * C + c, (part + Dc * x) * siluf_(z));
-    }
+    if (ok && nl == 0) st(out + (int64_t)t * C + c, (part + Dc * x) * siluf_(z));
   }
   if (ok) {
 #pragma unroll
@@ -140,23 +158,36 @@ __global__ __launch_bounds__(BT) void gdelta_scan_kernel(
   for (int i = 0; i < KD; ++i) S[i] = (col && i < d && init) ? sp[(int64_t)i * d + j] : 0.f;
   const int e = h * d + (col ? j : 0);
   const float w0e = ld(w0 + e), abe = ld(a_b + e), nwe = ld(norm_w + e);
-  for (int t = lo; t < hi; ++t) {
+  // the token's seven inputs of this column are fetched one token ahead, so their latency
+  // overlaps the previous token's arithmetic and barriers
+  float nk = 0.f, na = 0.f, nwl = 0.f, nr = 0.f, nv = 0.f, ng = 0.f;
+  auto fetch = [&](int t) {
+    if (!col || t >= hi) return;
     const T* pr = proj + (int64_t)t * p_stride;
-    const float kj = col ? ld(pr + HD + e) : 0.f;
+    nr = ld(pr + e);
+    nk = ld(pr + HD + e);
+    nv = ld(pr + 2 * HD + e);
+    ng = ld(pr + 3 * HD + e);
+    na = ld(pr + 4 * HD + e);
+    nwl = ld(wl + (int64_t)t * HD + e);
+  };
+  fetch(lo);
+  for (int t = lo; t < hi; ++t) {
+    const float kj = nk, aj = na, wlj = nwl, rj = nr, v = nv, gj = ng;
+    fetch(t + 1);
     const float ksum = block_sum<BT>(kj * kj, red);  // also fences the previous token's LDS reads
     if (col) {
       const float u = kj / sqrtf(ksum + 1e-6f);
-      const float a = sigmoidf_(ld(pr + 4 * HD + e) + abe);
-      sw[j] = expf(-DECAY_K * sigmoidf_(ld(wl + (int64_t)t * HD + e) + w0e));
+      const float a = sigmoidf_(aj + abe);
+      sw[j] = expf(-DECAY_K * sigmoidf_(wlj + w0e));
       sau[j] = a * u;
       su[j] = u;
       sk[j] = kj;
-      sr[j] = ld(pr + e);
+      sr[j] = rj;
     }
     __syncthreads();
     float o = 0.f;
     if (col) {
-      const float v = ld(pr + 2 * HD + e);
       float sa = 0.f;
 #pragma unroll
       for (int i = 0; i < KD; ++i)
@@ -169,10 +200,7 @@ __global__ __launch_bounds__(BT) void gdelta_scan_kernel(
         }
     }
     const float ss = block_sum<BT>(o * o, red);
-    if (col) {
-      const float g = sigmoidf_(ld(pr + 3 * HD + e));
-      st(out + (int64_t)t * HD + e, o / sqrtf(ss / (float)d + eps) * nwe * g);
-    }
+    if (col) st(out + (int64_t)t * HD + e, o / sqrtf(ss / (float)d + eps) * nwe * sigmoidf_(gj));
   }
   if (col) {
 #pragma unroll

@@ -98,7 +98,8 @@ def _time(r, pl, reps: int) -> float:
     return (time.perf_counter() - t0) / reps
 
 
-def run(tokens: int = 2048, batch: int = 32, n_layers: int = 4, reps: int = 5, device: str = "cuda") -> dict:
+def run(tokens: int = 2048, batch: int = 32, n_layers: int = 4, reps: int = 5, device: str = "cuda",
+        only: str = "") -> dict:
     import dataclasses
 
     from llmd_amd.engine.config import get_model_config
@@ -109,6 +110,8 @@ def run(tokens: int = 2048, batch: int = 32, n_layers: int = 4, reps: int = 5, d
     todo = [("latent+moe", stack_config(_attn(), n_layers), n_layers), ("mamba", stack_config(_mamba(), n_layers), n_layers),
             ("delta", stack_config(_delta(), n_layers), n_layers), ("deepseek-v2-lite (1 dense + moe layers)", ref, n_layers + 1)]
     for name, mc, L in todo:
+        if only and not name.startswith(only):
+            continue
         r = _runner(mc, tokens, batch, device)
         pre, dec = _plans(r, tokens, batch)
         tp, td = _time(r, pre, reps), _time(r, dec, reps * 4)
@@ -125,8 +128,9 @@ def main(argv=None):
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--layers", type=int, default=4)
     ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--only", default="", help="run the entries whose name starts with this")
     a = ap.parse_args(argv)
-    print(json.dumps(run(a.tokens, a.batch, a.layers, a.reps)), flush=True)
+    print(json.dumps(run(a.tokens, a.batch, a.layers, a.reps, only=a.only)), flush=True)
 
 
 if __name__ == "__main__":
