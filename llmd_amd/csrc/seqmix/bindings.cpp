@@ -19,6 +19,8 @@ void sm_latent_rope_cache(const void*, int64_t, const void*, int64_t, const void
                           int, int, int, int, int, const int64_t*, void*, void*, int, int, hipStream_t);
 int sm_latent_attention(const void*, const void*, const int*, int, int, const int*, const int*, float, int, int, int,
                         int, int, void*, int, hipStream_t);
+int sm_latent_attention_mfma(const void*, const void*, const int*, int, int, const int*, int, const int*, float, int,
+                             int, int, void*, hipStream_t);
 void sm_causal_conv_silu(const void*, int64_t, int, const void*, const void*, int, void*, const int*, const int*,
                          const int*, void*, int, int, int, hipStream_t);
 int sm_selective_scan(const void*, const void*, const void*, const float*, const void*, int64_t, int, int, const void*,
@@ -178,6 +180,27 @@ void latent_attention(Tensor q_abs, Tensor cache, Tensor tables, Tensor row_seq,
   TORCH_CHECK(rc == 0, "latent_attention: latent rank above 1024 or rows too wide for the LDS tile");
 }
 
+bool latent_attention_mfma(Tensor q_abs, Tensor cache, Tensor tables, Tensor items, Tensor row_len, double scale,
+                           int64_t R, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(q_abs));
+  TORCH_CHECK(q_abs.is_cuda() && q_abs.scalar_type() == torch::kBFloat16 && q_abs.dim() == 3 && q_abs.is_contiguous(),
+              "q_abs [T, H, Dk] bf16");
+  const int T = q_abs.size(0), H = q_abs.size(1), Dk = q_abs.size(2);
+  CHECK_ACT(cache, q_abs);
+  TORCH_CHECK(cache.dim() == 3 && cache.is_contiguous() && cache.size(2) == Dk && R >= 1 && R <= Dk, "cache");
+  CHECK_I32(tables);
+  CHECK_I32(items);
+  CHECK_I32(row_len);
+  TORCH_CHECK(tables.dim() == 2 && row_len.numel() == T && items.dim() == 2 && items.size(1) == 3, "tables");
+  CHECK_ACT(out, q_abs);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == (int64_t)T * H * R, "out [T, H, R]");
+  // the items are built by ops.seqmix.attention_items from the step's run lengths: rows inside [0, T),
+  // tokens * H <= 64
+  return sm_latent_attention_mfma(q_abs.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
+                                  cache.size(1), items.data_ptr<int>(), items.size(0), row_len.data_ptr<int>(),
+                                  (float)scale, H, R, Dk, out.data_ptr(), cur()) == 0;
+}
+
 void causal_conv_silu(Tensor xz, int64_t C, Tensor w, Tensor b, Tensor state, Tensor seq_start, Tensor seq_slot,
                       Tensor seq_init, int64_t max_q, Tensor out) {
   const c10::hip::OptionalHIPGuard g(dev_of(xz));
@@ -314,6 +337,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("softcap", &softcap);
   m.def("latent_rope_cache", &latent_rope_cache);
   m.def("latent_attention", &latent_attention);
+  m.def("latent_attention_mfma", &latent_attention_mfma);
   m.def("causal_conv_silu", &causal_conv_silu);
   m.def("selective_scan", &selective_scan);
   m.def("gdelta_scan", &gdelta_scan);

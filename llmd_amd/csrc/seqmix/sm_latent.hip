@@ -177,6 +177,161 @@ __global__ __launch_bounds__(NT) void latent_attention_kernel(
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// bf16 form on the matrix cores. A workgroup takes one work item: up to 64 (token, head) rows of
+// ONE sequence (consecutive tokens x all heads), 16 rows per wave. Keys stream through LDS in tiles
+// of 32: the tile row-major for the scores (S^T = K Q^T, v_mfma_f32_16x16x32_bf16, fp32
+// accumulation of exact bf16 products) and the latent part transposed for P x latent. Softmax is
+// fp32 per row; the weights P enter the second product as a bf16 pair (hi + lo, two MFMAs), which
+// keeps 16 mantissa bits of the fp32 weight. DkP = 32 NKS >= Dk and RP = 16 NCB >= R are the
+// padded sizes (zeros in LDS and in the query fragments).
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int MKT = 32;  // keys per tile
+
+template <int NKS, int NCB>
+__global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
+    const bf16_t* __restrict__ q_abs, const bf16_t* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
+    const int* __restrict__ items, const int* __restrict__ row_len, float scale, int H, int R, int Dk,
+    bf16_t* __restrict__ out) {
+  constexpr int DkP = 32 * NKS, RP = 16 * NCB;
+  constexpr int KS = DkP + 8, VS = MKT + 8, PS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
+  __shared__ __attribute__((aligned(16))) bf16_t sK[MKT * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t sVt[RP * VS];
+  __shared__ __attribute__((aligned(16))) bf16_t sPh[4 * 16 * PS];
+  __shared__ __attribute__((aligned(16))) bf16_t sPl[4 * 16 * PS];
+  const int seq = items[blockIdx.x * 3], tok0 = items[blockIdx.x * 3 + 1], ntok = items[blockIdx.x * 3 + 2];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, kq = lane >> 4;
+  // this lane's query row (as the B operand's column): item row 16 wave + r16
+  const int myrow = wave * 16 + r16;
+  const bool row_ok = myrow < ntok * H;
+  const int mytok = tok0 + (row_ok ? myrow / H : 0), myhead = row_ok ? myrow % H : 0;
+  const int mylen = row_ok ? row_len[mytok] : 0;
+  const int maxlen = row_len[tok0 + ntok - 1];  // the run's last token sees the most keys
+
+  bf16x8_t qf[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int d = ks * 32 + kq * 8 + i;
+      const bf16_t w = (row_ok && d < Dk) ? q_abs[((int64_t)mytok * H + myhead) * Dk + d] : (bf16_t)0;
+      qf[ks][i] = __builtin_bit_cast(__bf16, w);
+    }
+  }
+  f32x4_t o[NCB];
+#pragma unroll
+  for (int n = 0; n < NCB; ++n) o[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int* bt = tables + (int64_t)seq * W;
+  bf16_t* ph = sPh + wave * 16 * PS;
+  bf16_t* pl = sPl + wave * 16 * PS;
+  const bool vec = (Dk & 7) == 0;
+
+  for (int k0 = 0; k0 < maxlen; k0 += MKT) {
+    __syncthreads();  // the previous tile is no longer read
+    for (int e = threadIdx.x; e < MKT * (DkP / 8); e += NT) {
+      const int j = e / (DkP / 8), c = e - j * (DkP / 8);
+      const int key = k0 + j;
+      __attribute__((aligned(16))) bf16_t v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = 0;
+      if (key < maxlen) {
+        const bf16_t* src = cache + ((int64_t)bt[key / bs] * bs + (key % bs)) * Dk + c * 8;
+        if (vec && c * 8 + 8 <= Dk) {
+          *reinterpret_cast<u32x4_t*>(v) = *reinterpret_cast<const u32x4_t*>(src);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (c * 8 + i < Dk) v[i] = src[i];
+        }
+      }
+      *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = *reinterpret_cast<u32x4_t*>(v);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int d = c * 8 + i;
+        if (d < RP) sVt[d * VS + j] = d < R ? v[i] : (bf16_t)0;
+      }
+    }
+    __syncthreads();
+    // scores of this lane's row against keys k0 + 16 kb + 4 kq + r
+    float sc[2][4];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      f32x4_t a = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(&sK[(kb * 16 + r16) * KS + ks * 32 + kq * 8]);
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], a, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sc[kb][r] = (k0 + kb * 16 + kq * 4 + r < mylen) ? a[r] * scale : -INFINITY;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sc[kb][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    const float mref = (mn == -INFINITY) ? 0.f : mn;  // a row with no key yet
+    const float corr = expf(m - mref);
+    float psum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float pv = expf(sc[kb][r] - mref);
+        psum += pv;
+        const __bf16 hi = (__bf16)pv;
+        const __bf16 lo = (__bf16)(pv - (float)hi);
+        ph[r16 * PS + kb * 16 + kq * 4 + r] = __builtin_bit_cast(bf16_t, hi);
+        pl[r16 * PS + kb * 16 + kq * 4 + r] = __builtin_bit_cast(bf16_t, lo);
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = mn;
+    // the accumulators hold rows 4 kq + r: their correction comes from the lane that owns the row
+    float cr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, kq * 4 + r, 64);
+    __syncthreads();  // P of every wave is in LDS
+    const bf16x8_t pah = *reinterpret_cast<const bf16x8_t*>(&ph[r16 * PS + kq * 8]);
+    const bf16x8_t pal = *reinterpret_cast<const bf16x8_t*>(&pl[r16 * PS + kq * 8]);
+#pragma unroll
+    for (int n = 0; n < NCB; ++n) {
+      const bf16x8_t vb = *reinterpret_cast<const bf16x8_t*>(&sVt[(n * 16 + r16) * VS + kq * 8]);
+      f32x4_t acc = o[n];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[r] *= cr[r];
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pah, vb, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pal, vb, acc, 0, 0, 0);
+      o[n] = acc;
+    }
+  }
+  // o[n][r] = O[row 4 kq + r][column 16 n + r16]
+  float inv[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) inv[r] = 1.f / __shfl(l, kq * 4 + r, 64);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = wave * 16 + kq * 4 + r;
+    if (row >= ntok * H) continue;
+    const int64_t base = ((int64_t)(tok0 + row / H) * H + row % H) * R;
+#pragma unroll
+    for (int n = 0; n < NCB; ++n) {
+      const int col = n * 16 + r16;
+      if (col < R) st(out + base + col, o[n][r] * inv[r]);
+    }
+  }
+}
+
 template <typename T, int RC>
 int launch_attn(const void* q_abs, const void* cache, const int* tables, int W, int bs, const int* row_seq,
                 const int* row_len, float scale, int H, int R, int Dk, int T_rows, int QT, void* out,
@@ -236,6 +391,29 @@ int sm_latent_attention(const void* q_abs, const void* cache, const int* tables,
     if (rc <= 8) SM_GO(bf16_t, 8);
     if (rc <= 16) SM_GO(bf16_t, 16);
   }
+#undef SM_GO
+  return 1;
+}
+
+// bf16, matrix cores. items [n, 3] = (sequence, first token row, tokens), tokens * H <= 64.
+// Returns 0, or 1 when the sizes are outside the compiled forms (Dk > 576, R > 512, H > 64).
+int sm_latent_attention_mfma(const void* q_abs, const void* cache, const int* tables, int W, int bs, const int* items,
+                             int n_items, const int* row_len, float scale, int H, int R, int Dk, void* out,
+                             hipStream_t stream) {
+  if (n_items == 0) return 0;
+  const int nks = (Dk + 31) / 32, ncb = (R + 15) / 16;
+  if (H > 64) return 1;
+#define SM_GO(NKS, NCB)                                                                                           \
+  {                                                                                                                 \
+    hipLaunchKernelGGL((latent_attention_mfma_kernel<NKS, NCB>), dim3(n_items), dim3(NT), 0, stream,               \
+                       (const bf16_t*)q_abs, (const bf16_t*)cache, tables, W, bs, items, row_len, scale, H, R, Dk,  \
+                       (bf16_t*)out);                                                                               \
+    return 0;                                                                                                       \
+  }
+  if (nks <= 3 && ncb <= 4) SM_GO(3, 4)
+  if (nks <= 6 && ncb <= 8) SM_GO(6, 8)
+  if (nks <= 10 && ncb <= 16) SM_GO(10, 16)
+  if (nks <= 18 && ncb <= 32) SM_GO(18, 32)
 #undef SM_GO
   return 1;
 }

@@ -27,6 +27,26 @@ class SeqMeta:
     tables: torch.Tensor             # [n, W] int32 block tables
     max_len: int = 0                 # longest context of the step
     max_q: int = 0                   # longest run of the step
+    q_lens: Optional[list] = None    # host copy of the run lengths
+    _items: Optional[dict] = None    # tokens per item -> [n, 3] int32 work items (attention_items)
+
+    def attention_items(self, tokens_per_item: int) -> torch.Tensor:
+        """Work items (sequence, first token row, tokens) of the matrix-core attention kernel: every
+        run cut into pieces of at most ``tokens_per_item`` tokens. Built once per step and size."""
+        if self._items is None:
+            self._items = {}
+        it = self._items.get(tokens_per_item)
+        if it is None:
+            rows, t0 = [], 0
+            for s, n in enumerate(self.q_lens):
+                for a in range(0, n, tokens_per_item):
+                    rows.append((s, t0 + a, min(tokens_per_item, n - a)))
+                t0 += n
+            it = torch.tensor(rows, dtype=torch.int32).view(-1, 3)
+            if self.tables.is_cuda:
+                it = it.pin_memory().to(self.tables.device, non_blocking=True)
+            self._items[tokens_per_item] = it
+        return it
 
 
 @dataclass

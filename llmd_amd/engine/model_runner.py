@@ -829,7 +829,8 @@ class ModelRunner:
         return SeqMeta(num_seqs=n, seq_start=sd[o[0]:o[1]], seq_slot=sd[o[1]:o[2]], seq_init=sd[o[2]:o[3]],
                        row_seq=sd[o[3]:o[4]], row_len=sd[o[4]:o[5]],
                        tables=torch.from_numpy(np.ascontiguousarray(tables)).to(dev, non_blocking=True),
-                       max_len=int(row_len.max()) if T else 0, max_q=int(ql.max()) if n else 0)
+                       max_len=int(row_len.max()) if T else 0, max_q=int(ql.max()) if n else 0,
+                       q_lens=ql.tolist())
 
     @torch.no_grad()
     def forward_logits(self, so: SchedulerOutput, block_tables: dict, rows: list[int]):

@@ -85,7 +85,7 @@ class LatentAttention(torch.nn.Module):
         qn = q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1)                       # [H, T, dn]
         q_abs[:, :, :R].copy_(torch.bmm(qn, self.uk.view(H, dn, R)).transpose(0, 1))
         o_lat = sm.latent_attention(q_abs, self.cache, s.tables, s.row_seq, s.row_len, self.scale, R,
-                                    rows_per_group=4 if s.max_q > 1 else 1)
+                                    rows_per_group=4 if s.max_q > 1 else 1, seq=s)
         o = torch.bmm(o_lat.transpose(0, 1), self.uv.view(H, self.dv, R).transpose(1, 2))  # [H, T, dv]
         return self.o(o.transpose(0, 1).reshape(T, H * self.dv))
 

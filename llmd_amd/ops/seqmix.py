@@ -84,15 +84,27 @@ def latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dim
                                q_abs)
 
 
-def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: int, rows_per_group: int = 1):
+MFMA_ATTENTION = os.environ.get("LLMD_LATENT_MFMA", "1") == "1"
+
+
+def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: int, rows_per_group: int = 1,
+                     seq=None):
     """Causal softmax attention of absorbed queries [T, H, R + dr] over the paged latent cache
     [blocks, bs, R + dr]; row t sees the first row_len[t] keys of sequence row_seq[t].
-    Returns the latent outputs [T, H, R]. ``rows_per_group`` (1 or 4): consecutive rows that share
-    a workgroup's key tiles - 4 for steps with prompt portions, 1 for decode-only steps."""
+    Returns the latent outputs [T, H, R].
+
+    bfloat16 with the step's ``seq`` description (engine/attn_meta.py SeqMeta): the matrix-core
+    kernel over work items of up to 64 (token, head) rows of one sequence (R + dr <= 576, R <= 512,
+    H <= 64). Otherwise (float32, other sizes) the fp32 FMA kernel; ``rows_per_group`` (1 or 4) is
+    its number of consecutive rows that share a workgroup's key tiles."""
     T, H, _ = q_abs.shape
     out = torch.empty(T, H, R, dtype=q_abs.dtype, device=q_abs.device)
     if not q_abs.is_cuda:
         return ref.latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out)
+    if MFMA_ATTENTION and seq is not None and q_abs.dtype == torch.bfloat16 and H <= 64:
+        items = seq.attention_items(max(1, 64 // H))
+        if native().latent_attention_mfma(q_abs, cache, tables, items, row_len, float(scale), R, out):
+            return out
     native().latent_attention(q_abs, cache, tables, row_seq, row_len, float(scale), R, int(rows_per_group), out)
     return out
 

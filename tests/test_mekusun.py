@@ -288,3 +288,41 @@ def test_config_reads_sizes_from_file_and_shapes(tmp_path):
     assert mc.layer_specs[1]["mixer"]["decay_rank"] == 11
     assert mc.embedding_scale == 3.0 and mc.logit_softcap == 20.0
     assert os.path.exists(os.path.join(path, "model.safetensors"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,R,dr", [(3, 40, 8), (5, 24, 12), (6, 64, 16), (16, 512, 64), (2, 100, 30)])
+def test_matrix_core_attention_matches_fp32(H, R, dr):
+    """bfloat16 attention on the matrix cores against the fp32 kernel on the same (bf16-rounded)
+    inputs: a prompt portion that continues a context, a whole prompt and two decode rows in one
+    step, over shuffled pages; sizes that need padding to the MFMA shapes included."""
+    from llmd_amd.engine.attn_meta import SeqMeta
+    from llmd_amd.ops import seqmix as sm
+
+    dev, bs, Dk = "cuda", 64, R + dr
+    g = torch.Generator().manual_seed(H * 1000 + R)
+    # (context before the run, run length): decodes first, then the portions
+    runs = [(130, 1), (63, 1), (70, 37), (0, 90)]
+    nblk = [-(-(c + n) // bs) for c, n in runs]
+    perm = torch.randperm(sum(nblk) + 2, generator=g)
+    tables = torch.zeros(len(runs), max(nblk), dtype=torch.int32)
+    o = 0
+    for i, k in enumerate(nblk):
+        tables[i, :k] = perm[o:o + k]
+        o += k
+    cache = (torch.randn(sum(nblk) + 2, bs, Dk, generator=g) * 0.5).to(torch.bfloat16)
+    T = sum(n for _, n in runs)
+    q = (torch.randn(T, H, Dk, generator=g) * 0.7).to(torch.bfloat16)
+    row_seq = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, (_, n) in enumerate(runs)])
+    row_len = torch.cat([torch.arange(c + 1, c + n + 1, dtype=torch.int32) for c, n in runs])
+    start = torch.tensor([0] + list(torch.tensor([n for _, n in runs]).cumsum(0)), dtype=torch.int32)
+    seq = SeqMeta(num_seqs=len(runs), seq_start=start.to(dev), seq_slot=torch.zeros(4, dtype=torch.int32, device=dev),
+                  seq_init=torch.zeros(4, dtype=torch.int32, device=dev), row_seq=row_seq.to(dev),
+                  row_len=row_len.to(dev), tables=tables.to(dev), max_len=int(row_len.max()), max_q=90,
+                  q_lens=[n for _, n in runs])
+    scale = Dk ** -0.5
+    fast = sm.latent_attention(q.to(dev), cache.to(dev), seq.tables, seq.row_seq, seq.row_len, scale, R, 4, seq=seq)
+    slow = sm.latent_attention(q.float().to(dev), cache.float().to(dev), seq.tables, seq.row_seq, seq.row_len, scale, R, 4)
+    assert fast.dtype == torch.bfloat16
+    err = (fast.float() - slow).abs().max() / slow.abs().max()
+    assert float(err) < 8e-3, float(err)
