@@ -140,6 +140,114 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
   }
 }
 
+
+// bf16 on the matrix cores: 64 rows x 128 columns per workgroup, K stepped by 64 through LDS
+// (next step's global loads in flight during the MFMAs). Wave (wm, wn) owns rows 32 wm.. and
+// columns 64 wn.. as 2 x 4 fragments of v_mfma_f32_16x16x32_bf16; fp32 accumulation in a fixed
+// K order. Needs K % 8 == 0 and 16-byte aligned rows (vector loads).
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int MBN = 128, MBK = 64, MLS = MBK + 8;  // LDS row stride 144 B
+
+template <bool GELU>
+__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __restrict__ A, int64_t a_stride, int kdiv,
+                                                            const int* __restrict__ slot_row,
+                                                            const int* __restrict__ tile_e,
+                                                            const bf16_t* __restrict__ Wt, int N, int K,
+                                                            bf16_t* __restrict__ Cout) {
+  const int e = tile_e[blockIdx.x];
+  if (e < 0) return;
+  __shared__ __attribute__((aligned(16))) bf16_t sA[TM * MLS];
+  __shared__ __attribute__((aligned(16))) bf16_t sB[MBN * MLS];
+  __shared__ int srow[TM];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int slot0 = blockIdx.x * TM, n0 = blockIdx.y * MBN;
+  if (tid < TM) {
+    const int p = slot_row[slot0 + tid];
+    srow[tid] = p < 0 ? -1 : (kdiv > 0 ? p / kdiv : slot0 + tid);
+  }
+  __syncthreads();
+  const bf16_t* We = Wt + (int64_t)e * N * K;
+  // staging: A 64 rows x 8 chunks of 16 B (2 per thread), B 128 x 8 (4 per thread)
+  u32x4_t ra[2], rb[4];
+  auto load = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c = tid + 256 * i, r = c >> 3, ch = c & 7;
+      u32x4_t v = {0, 0, 0, 0};
+      const int ar = srow[r];
+      if (ar >= 0 && k0 + ch * 8 < K) v = *reinterpret_cast<const u32x4_t*>(A + (int64_t)ar * a_stride + k0 + ch * 8);
+      ra[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + 256 * i, r = c >> 3, ch = c & 7;
+      u32x4_t v = {0, 0, 0, 0};
+      if (n0 + r < N && k0 + ch * 8 < K) v = *reinterpret_cast<const u32x4_t*>(We + (int64_t)(n0 + r) * K + k0 + ch * 8);
+      rb[i] = v;
+    }
+  };
+  auto store = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c = tid + 256 * i;
+      *reinterpret_cast<u32x4_t*>(&sA[(c >> 3) * MLS + (c & 7) * 8]) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + 256 * i;
+      *reinterpret_cast<u32x4_t*>(&sB[(c >> 3) * MLS + (c & 7) * 8]) = rb[i];
+    }
+  };
+  f32x4_t acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int r16 = lane & 15, kq = lane >> 4;
+  const int nk = (K + MBK - 1) / MBK;
+  load(0);
+  for (int kt = 0; kt < nk; ++kt) {
+    __syncthreads();  // the previous step's fragments are read
+    store();
+    __syncthreads();
+    if (kt + 1 < nk) load((kt + 1) * MBK);
+#pragma unroll
+    for (int ks = 0; ks < MBK / 32; ++ks) {
+      bf16x8_t af[2], bfr[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        af[i] = *reinterpret_cast<const bf16x8_t*>(&sA[(wm * 32 + i * 16 + r16) * MLS + ks * 32 + kq * 8]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        bfr[j] = *reinterpret_cast<const bf16x8_t*>(&sB[(wn * 64 + j * 16 + r16) * MLS + ks * 32 + kq * 8]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  // acc[i][j][r] = C[row 32 wm + 16 i + 4 kq + r][column 64 wn + 16 j + r16]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = wm * 32 + i * 16 + kq * 4 + r;
+      if (srow[row] < 0) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + wn * 64 + j * 16 + r16;
+        if (n >= N) continue;
+        float v = acc[i][j][r];
+        if (GELU) v = 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
+        st(Cout + (int64_t)(slot0 + row) * N + n, v);
+      }
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ pair_slot,
                                                           const float* __restrict__ w, int k, int d,
@@ -169,6 +277,16 @@ void sm_moe_group(const int* ids, int n, int E, int* slot_row, int* tile_e, int*
 
 void sm_moe_gemm(const void* A, int64_t a_stride, int kdiv, const int* slot_row, const int* tile_e, const void* W,
                  int N, int K, void* C, int max_tiles, int gelu, int f32, hipStream_t stream) {
+  if (!f32 && K % 8 == 0 && a_stride % 8 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0) {
+    const dim3 g2(max_tiles, (N + MBN - 1) / MBN);
+    if (gelu)
+      hipLaunchKernelGGL((moe_gemm_mfma_kernel<true>), g2, dim3(256), 0, stream, (const bf16_t*)A, a_stride, kdiv,
+                         slot_row, tile_e, (const bf16_t*)W, N, K, (bf16_t*)C);
+    else
+      hipLaunchKernelGGL((moe_gemm_mfma_kernel<false>), g2, dim3(256), 0, stream, (const bf16_t*)A, a_stride, kdiv,
+                         slot_row, tile_e, (const bf16_t*)W, N, K, (bf16_t*)C);
+    return;
+  }
   const dim3 grid(max_tiles, (N + TN - 1) / TN);
 #define SM_GO(TYPE, G)                                                                                          \
   hipLaunchKernelGGL((moe_gemm_kernel<TYPE, G>), grid, dim3(256), 0, stream, (const TYPE*)A, a_stride, kdiv,   \

@@ -144,7 +144,7 @@ __global__ __launch_bounds__(BT) void gdelta_scan_kernel(
     const T* __restrict__ a_b, const T* __restrict__ norm_w, float eps, int H, int d, float* __restrict__ state,
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot, const int* __restrict__ seq_init,
     T* __restrict__ out) {
-  __shared__ float sw[KD], sau[KD], su[KD], sk[KD], sr[KD];
+  __shared__ __attribute__((aligned(16))) float sw[KD], sau[KD], su[KD], sk[KD], sr[KD];
   __shared__ float red[BT / 64];
   const int h = blockIdx.x, s = blockIdx.y;
   const int j = threadIdx.x;
@@ -156,6 +156,7 @@ __global__ __launch_bounds__(BT) void gdelta_scan_kernel(
   const bool init = seq_init[s] != 0;
 #pragma unroll
   for (int i = 0; i < KD; ++i) S[i] = (col && i < d && init) ? sp[(int64_t)i * d + j] : 0.f;
+  for (int i = d + j; i < KD; i += BT) sw[i] = sau[i] = su[i] = sk[i] = sr[i] = 0.f;
   const int e = h * d + (col ? j : 0);
   const float w0e = ld(w0 + e), abe = ld(a_b + e), nwe = ld(norm_w + e);
   // the token's seven inputs of this column are fetched one token ahead, so their latency
@@ -188,16 +189,30 @@ __global__ __launch_bounds__(BT) void gdelta_scan_kernel(
     __syncthreads();
     float o = 0.f;
     if (col) {
+      // the key-side vectors come as 16-byte LDS broadcasts; entries beyond d are zero
+      // (written below), so whole groups of four need no bound
       float sa = 0.f;
 #pragma unroll
-      for (int i = 0; i < KD; ++i)
-        if (i < d) sa += su[i] * S[i];
-#pragma unroll
-      for (int i = 0; i < KD; ++i)
+      for (int i = 0; i < KD; i += 4) {
         if (i < d) {
-          S[i] = sw[i] * S[i] - sau[i] * sa + sk[i] * v;
-          o += S[i] * sr[i];
+          const float4 u4 = *reinterpret_cast<const float4*>(&su[i]);
+          sa += u4.x * S[i] + u4.y * S[i + 1] + u4.z * S[i + 2] + u4.w * S[i + 3];
         }
+      }
+#pragma unroll
+      for (int i = 0; i < KD; i += 4) {
+        if (i < d) {
+          const float4 w4 = *reinterpret_cast<const float4*>(&sw[i]);
+          const float4 a4 = *reinterpret_cast<const float4*>(&sau[i]);
+          const float4 k4 = *reinterpret_cast<const float4*>(&sk[i]);
+          const float4 r4 = *reinterpret_cast<const float4*>(&sr[i]);
+          S[i] = w4.x * S[i] - a4.x * sa + k4.x * v;
+          S[i + 1] = w4.y * S[i + 1] - a4.y * sa + k4.y * v;
+          S[i + 2] = w4.z * S[i + 2] - a4.z * sa + k4.z * v;
+          S[i + 3] = w4.w * S[i + 3] - a4.w * sa + k4.w * v;
+          o += S[i] * r4.x + S[i + 1] * r4.y + S[i + 2] * r4.z + S[i + 3] * r4.w;
+        }
+      }
     }
     const float ss = block_sum<BT>(o * o, red);
     if (col) st(out + (int64_t)t * HD + e, o / sqrtf(ss / (float)d + eps) * nwe * sigmoidf_(gj));

@@ -326,3 +326,29 @@ def test_matrix_core_attention_matches_fp32(H, R, dr):
     assert fast.dtype == torch.bfloat16
     err = (fast.float() - slow).abs().max() / slow.abs().max()
     assert float(err) < 8e-3, float(err)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,d,F,E,k", [(70, 48, 24, 5, 2), (300, 256, 200, 16, 3), (9, 64, 72, 4, 4), (33, 50, 30, 3, 1)])
+def test_expert_gemm_bf16_matches_fp32(T, d, F, E, k):
+    """The bfloat16 expert feed-forward (matrix cores where rows are 16-byte aligned, the FMA
+    kernel otherwise) against the float32 kernels on the same bf16-rounded inputs."""
+    from llmd_amd.ops import seqmix as sm
+
+    g = torch.Generator().manual_seed(T + d)
+    h = torch.randn(T, d, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(E, F, d, generator=g) / math.sqrt(d)).to(torch.bfloat16)
+    w2 = (torch.randn(E, d, F, generator=g) / math.sqrt(F)).to(torch.bfloat16)
+    logits = torch.randn(T, E, generator=g).cuda()
+    ids, w = sm.moe_route(logits, k)
+    top, idx = logits.topk(k, -1)
+    assert torch.equal(ids.long(), idx) and torch.allclose(w, torch.softmax(top, -1), atol=1e-6)
+    fast = sm.moe_ffn(h.cuda(), ids, w, w1.cuda(), w2.cuda())
+    slow = sm.moe_ffn(h.float().cuda(), ids, w, w1.float().cuda(), w2.float().cuda())
+    want = torch.zeros(T, d, dtype=torch.float64)
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            want[t] += float(w[t, j]) * (oracle.gelu_erf(h[t].double() @ w1[e].double().T) @ w2[e].double().T)
+    assert float((slow.cpu().double() - want).abs().max() / want.abs().max()) < 1e-5
+    assert float((fast.float() - slow).abs().max() / slow.abs().max()) < 2e-2
