@@ -20,7 +20,7 @@ void sm_latent_rope_cache(const void*, int64_t, const void*, int64_t, const void
 int sm_latent_attention(const void*, const void*, const int*, int, int, const int*, const int*, float, int, int, int,
                         int, int, void*, int, hipStream_t);
 int sm_latent_attention_mfma(const void*, const void*, const int*, int, int, const int*, int, const int*, float, int,
-                             int, int, void*, hipStream_t);
+                             int, int, void*, int, int, float*, float*, hipStream_t);
 void sm_causal_conv_silu(const void*, int64_t, int, const void*, const void*, int, void*, const int*, const int*,
                          const int*, void*, int, int, int, hipStream_t);
 int sm_selective_scan(const void*, const void*, const void*, const float*, const void*, int64_t, int, int, const void*,
@@ -181,7 +181,8 @@ void latent_attention(Tensor q_abs, Tensor cache, Tensor tables, Tensor row_seq,
 }
 
 bool latent_attention_mfma(Tensor q_abs, Tensor cache, Tensor tables, Tensor items, Tensor row_len, double scale,
-                           int64_t R, Tensor out) {
+                           int64_t R, Tensor out, int64_t nsplit, int64_t split_keys, c10::optional<Tensor> part_o,
+                           c10::optional<Tensor> part_ml) {
   const c10::hip::OptionalHIPGuard g(dev_of(q_abs));
   TORCH_CHECK(q_abs.is_cuda() && q_abs.scalar_type() == torch::kBFloat16 && q_abs.dim() == 3 && q_abs.is_contiguous(),
               "q_abs [T, H, Dk] bf16");
@@ -196,9 +197,21 @@ bool latent_attention_mfma(Tensor q_abs, Tensor cache, Tensor tables, Tensor ite
   TORCH_CHECK(out.is_contiguous() && out.numel() == (int64_t)T * H * R, "out [T, H, R]");
   // the items are built by ops.seqmix.attention_items from the step's run lengths: rows inside [0, T),
   // tokens * H <= 64
+  float *po = nullptr, *pm = nullptr;
+  TORCH_CHECK(nsplit >= 1 && nsplit <= 1024, "key ranges per item");
+  if (nsplit > 1) {
+    TORCH_CHECK(split_keys >= 32 && split_keys % 32 == 0, "keys per range: a multiple of 32");
+    TORCH_CHECK(part_o.has_value() && part_ml.has_value(), "split step without workspace");
+    CHECK_F32(*part_o);
+    CHECK_F32(*part_ml);
+    TORCH_CHECK(part_o->numel() >= items.size(0) * nsplit * 64 * R && part_ml->numel() >= items.size(0) * nsplit * 128,
+                "workspace too small");
+    po = part_o->data_ptr<float>();
+    pm = part_ml->data_ptr<float>();
+  }
   return sm_latent_attention_mfma(q_abs.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
                                   cache.size(1), items.data_ptr<int>(), items.size(0), row_len.data_ptr<int>(),
-                                  (float)scale, H, R, Dk, out.data_ptr(), cur()) == 0;
+                                  (float)scale, H, R, Dk, out.data_ptr(), nsplit, split_keys, po, pm, cur()) == 0;
 }
 
 void causal_conv_silu(Tensor xz, int64_t C, Tensor w, Tensor b, Tensor state, Tensor seq_start, Tensor seq_slot,

@@ -196,7 +196,7 @@ template <int NKS, int NCB>
 __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ q_abs, const bf16_t* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
     const int* __restrict__ items, const int* __restrict__ row_len, float scale, int H, int R, int Dk,
-    bf16_t* __restrict__ out) {
+    bf16_t* __restrict__ out, int split_keys, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int DkP = 32 * NKS, RP = 16 * NCB;
   constexpr int KS = DkP + 8, VS = MKT + 8, PS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
   __shared__ __attribute__((aligned(16))) bf16_t sK[MKT * KS];
@@ -232,7 +232,11 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
   bf16_t* pl = sPl + wave * 16 * PS;
   const bool vec = (Dk & 7) == 0;
 
-  for (int k0 = 0; k0 < maxlen; k0 += MKT) {
+  // decode steps split a row's keys over blockIdx.y: this workgroup takes [kbeg, kend)
+  const int nsplit = gridDim.y;
+  const int kbeg = nsplit > 1 ? blockIdx.y * split_keys : 0;
+  const int kend = nsplit > 1 ? min(maxlen, kbeg + split_keys) : maxlen;
+  for (int k0 = kbeg; k0 < kend; k0 += MKT) {
     __syncthreads();  // the previous tile is no longer read
     for (int e = threadIdx.x; e < MKT * (DkP / 8); e += NT) {
       const int j = e / (DkP / 8), c = e - j * (DkP / 8);
@@ -240,7 +244,7 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
       __attribute__((aligned(16))) bf16_t v[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = 0;
-      if (key < maxlen) {
+      if (key < kend) {
         const bf16_t* src = cache + ((int64_t)bt[key / bs] * bs + (key % bs)) * Dk + c * 8;
         if (vec && c * 8 + 8 <= Dk) {
           *reinterpret_cast<u32x4_t*>(v) = *reinterpret_cast<const u32x4_t*>(src);
@@ -269,7 +273,8 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
         a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], a, 0, 0, 0);
       }
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sc[kb][r] = (k0 + kb * 16 + kq * 4 + r < mylen) ? a[r] * scale : -INFINITY;
+      for (int r = 0; r < 4; ++r)
+        sc[kb][r] = (k0 + kb * 16 + kq * 4 + r < min(mylen, kend)) ? a[r] * scale : -INFINITY;
     }
     float mx = -INFINITY;
 #pragma unroll
@@ -316,6 +321,24 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
     }
   }
   // o[n][r] = O[row 4 kq + r][column 16 n + r16]
+  if (nsplit > 1) {
+    // partial result of this key range: unnormalised o, with the row's running max and sum
+    const int64_t pbase = ((int64_t)blockIdx.x * nsplit + blockIdx.y) * 64;
+    if (kq == 0) {
+      part_ml[(pbase + myrow) * 2] = m;
+      part_ml[(pbase + myrow) * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = wave * 16 + kq * 4 + r;
+#pragma unroll
+      for (int n = 0; n < NCB; ++n) {
+        const int col = n * 16 + r16;
+        if (col < R) part_o[(pbase + row) * R + col] = o[n][r];
+      }
+    }
+    return;
+  }
   float inv[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) inv[r] = 1.f / __shfl(l, kq * 4 + r, 64);
@@ -329,6 +352,32 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
       const int col = n * 16 + r16;
       if (col < R) st(out + base + col, o[n][r] * inv[r]);
     }
+  }
+}
+
+// Merge the key-range partials of a split step: out = sum_y e^(m_y - M) o_y / sum_y e^(m_y - M) l_y.
+__global__ __launch_bounds__(NT) void latent_attention_merge_kernel(const int* __restrict__ items, int nsplit,
+                                                                   const float* __restrict__ part_o,
+                                                                   const float* __restrict__ part_ml, int H, int R,
+                                                                   bf16_t* __restrict__ out) {
+  const int item = blockIdx.x, row = blockIdx.y;
+  const int tok0 = items[item * 3 + 1], ntok = items[item * 3 + 2];
+  if (row >= ntok * H) return;
+  float M = -INFINITY;
+  for (int y = 0; y < nsplit; ++y) M = fmaxf(M, part_ml[(((int64_t)item * nsplit + y) * 64 + row) * 2]);
+  float L = 0.f;
+  for (int y = 0; y < nsplit; ++y) {
+    const float* ml = part_ml + (((int64_t)item * nsplit + y) * 64 + row) * 2;
+    L += expf(ml[0] - M) * ml[1];  // an empty range has m = -inf, l = 0
+  }
+  const int64_t obase = ((int64_t)(tok0 + row / H) * H + row % H) * R;
+  for (int c = threadIdx.x; c < R; c += NT) {
+    float a = 0.f;
+    for (int y = 0; y < nsplit; ++y) {
+      const int64_t pb = ((int64_t)item * nsplit + y) * 64 + row;
+      a += expf(part_ml[pb * 2] - M) * part_o[pb * R + c];
+    }
+    st(out + obase + c, a / L);
   }
 }
 
@@ -396,26 +445,30 @@ int sm_latent_attention(const void* q_abs, const void* cache, const int* tables,
 }
 
 // bf16, matrix cores. items [n, 3] = (sequence, first token row, tokens), tokens * H <= 64.
+// nsplit > 1: every item's keys are cut into nsplit ranges of split_keys (a multiple of 32) that
+// run as separate workgroups; part_o [n * nsplit * 64 * R] and part_ml [n * nsplit * 64 * 2] fp32
+// hold their partial results and a second kernel merges them.
 // Returns 0, or 1 when the sizes are outside the compiled forms (Dk > 576, R > 512, H > 64).
 int sm_latent_attention_mfma(const void* q_abs, const void* cache, const int* tables, int W, int bs, const int* items,
                              int n_items, const int* row_len, float scale, int H, int R, int Dk, void* out,
-                             hipStream_t stream) {
+                             int nsplit, int split_keys, float* part_o, float* part_ml, hipStream_t stream) {
   if (n_items == 0) return 0;
   const int nks = (Dk + 31) / 32, ncb = (R + 15) / 16;
-  if (H > 64) return 1;
-#define SM_GO(NKS, NCB)                                                                                           \
-  {                                                                                                                 \
-    hipLaunchKernelGGL((latent_attention_mfma_kernel<NKS, NCB>), dim3(n_items), dim3(NT), 0, stream,               \
-                       (const bf16_t*)q_abs, (const bf16_t*)cache, tables, W, bs, items, row_len, scale, H, R, Dk,  \
-                       (bf16_t*)out);                                                                               \
-    return 0;                                                                                                       \
-  }
-  if (nks <= 3 && ncb <= 4) SM_GO(3, 4)
-  if (nks <= 6 && ncb <= 8) SM_GO(6, 8)
-  if (nks <= 10 && ncb <= 16) SM_GO(10, 16)
-  if (nks <= 18 && ncb <= 32) SM_GO(18, 32)
+  if (H > 64 || nks > 18 || ncb > 32) return 1;
+  const dim3 grid(n_items, nsplit);
+#define SM_GO(NKS, NCB)                                                                                            \
+  hipLaunchKernelGGL((latent_attention_mfma_kernel<NKS, NCB>), grid, dim3(NT), 0, stream, (const bf16_t*)q_abs,     \
+                     (const bf16_t*)cache, tables, W, bs, items, row_len, scale, H, R, Dk, (bf16_t*)out, split_keys, \
+                     part_o, part_ml)
+  if (nks <= 3 && ncb <= 4) SM_GO(3, 4);
+  else if (nks <= 6 && ncb <= 8) SM_GO(6, 8);
+  else if (nks <= 10 && ncb <= 16) SM_GO(10, 16);
+  else SM_GO(18, 32);
 #undef SM_GO
-  return 1;
+  if (nsplit > 1)
+    hipLaunchKernelGGL(latent_attention_merge_kernel, dim3(n_items, 64), dim3(NT), 0, stream, items, nsplit, part_o,
+                       part_ml, H, R, (bf16_t*)out);
+  return 0;
 }
 
 }  // extern "C"

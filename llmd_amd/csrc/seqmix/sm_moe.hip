@@ -47,6 +47,58 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   for (int j = 0; j < k; ++j) ow[j] /= s;
 }
 
+// One wave per token, lanes over experts (E <= 512: up to 8 logits per lane in registers): k rounds
+// of a wave-wide arg-max over the logits not yet chosen, ties to the lower index.
+__global__ __launch_bounds__(256) void moe_route_wave_kernel(const float* __restrict__ logits, int E, int k,
+                                                             int* __restrict__ ids, float* __restrict__ w, int T) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (t >= T) return;
+  const float* z = logits + (int64_t)t * E;
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < E ? z[e] : -INFINITY;
+  }
+  float m0 = 0.f, sum = 0.f, mine = 0.f;  // lane j keeps the j-th chosen weight
+  int mine_id = 0;
+  unsigned taken = 0;  // bit i: this lane's logit i is already chosen
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E && !(taken >> i & 1u) && (bi == 0x7fffffff || v[i] > best)) {
+        best = v[i];
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > best || (ob == best && oi < bi))) {
+        best = ob;
+        bi = oi;
+      }
+    }
+    if (j == 0) m0 = best;
+    const float p = expf(best - m0);
+    sum += p;
+    if (lane == j) {
+      mine = p;
+      mine_id = bi;
+    }
+    if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
+  }
+  if (lane < k) {
+    ids[(int64_t)t * k + lane] = mine_id;
+    w[(int64_t)t * k + lane] = mine / sum;
+  }
+}
+
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int n, int E,
                                                          int* __restrict__ slot_row, int* __restrict__ tile_e,
                                                          int* __restrict__ pair_slot, int max_tiles) {
@@ -266,6 +318,10 @@ extern "C" {
 
 void sm_moe_route(const float* logits, int E, int k, int* ids, float* w, int T, hipStream_t stream) {
   if (T == 0) return;
+  if (E <= 512 && k <= 64) {
+    hipLaunchKernelGGL(moe_route_wave_kernel, dim3((T + 3) / 4), dim3(256), 0, stream, logits, E, k, ids, w, T);
+    return;
+  }
   hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, stream, logits, E, k, ids, w, T);
 }
 

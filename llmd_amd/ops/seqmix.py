@@ -103,7 +103,18 @@ def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: in
         return ref.latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out)
     if MFMA_ATTENTION and seq is not None and q_abs.dtype == torch.bfloat16 and H <= 64:
         items = seq.attention_items(max(1, 64 // H))
-        if native().latent_attention_mfma(q_abs, cache, tables, items, row_len, float(scale), R, out):
+        nsplit, split, po, pm = 1, 0, None, None
+        if seq.max_q == 1 and seq.max_len > 256:
+            # decode-only step: cut the keys into ranges so that items x ranges fill the chip
+            n = items.shape[0]
+            nsplit = max(1, min(-(-512 // n), seq.max_len // 128))
+            split = -(-seq.max_len // (nsplit * 32)) * 32
+            nsplit = -(-seq.max_len // split)
+            if nsplit > 1:
+                po = torch.empty(n * nsplit * 64 * R, dtype=torch.float32, device=q_abs.device)
+                pm = torch.empty(n * nsplit * 128, dtype=torch.float32, device=q_abs.device)
+        if native().latent_attention_mfma(q_abs, cache, tables, items, row_len, float(scale), R, out, nsplit, split,
+                                          po, pm):
             return out
     native().latent_attention(q_abs, cache, tables, row_seq, row_len, float(scale), R, int(rows_per_group), out)
     return out

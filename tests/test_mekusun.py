@@ -258,6 +258,23 @@ def test_greedy_generation_through_the_scheduler(tmp_path, device):
     assert eng.bm.slots.num_free() == 2
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("E,k", [(5, 2), (64, 6), (130, 8), (16, 16), (600, 3)])
+def test_router_top_k(E, k):
+    from llmd_amd.ops import seqmix as sm
+
+    g = torch.Generator().manual_seed(E)
+    z = torch.randn(37, E, generator=g)
+    z[3, 1] = z[3, 0] = z[3].max() + 1.0          # a tie: the lower index comes first
+    ids, w = sm.moe_route(z.cuda(), k)
+    order = sorted(range(E), key=lambda e: (-float(z[3, e]), e))[:k]
+    assert ids[3].tolist() == order
+    top, idx = z.topk(k, -1)
+    assert torch.equal(ids.cpu().long().sort(-1).values, idx.sort(-1).values)
+    assert torch.allclose(w.cpu().sum(-1), torch.ones(37), atol=1e-6)
+    assert torch.allclose(w.cpu().sort(-1, descending=True).values, torch.softmax(top, -1), atol=1e-6)
+
+
 def test_state_slots_and_block_manager():
     from llmd_amd import _rt_loader
     from llmd_amd.engine.state_cache import StatefulBlockManager
@@ -291,8 +308,9 @@ def test_config_reads_sizes_from_file_and_shapes(tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("decode_only", [False, True], ids=["mixed-step", "decode-step"])
 @pytest.mark.parametrize("H,R,dr", [(3, 40, 8), (5, 24, 12), (6, 64, 16), (16, 512, 64), (2, 100, 30)])
-def test_matrix_core_attention_matches_fp32(H, R, dr):
+def test_matrix_core_attention_matches_fp32(H, R, dr, decode_only):
     """bfloat16 attention on the matrix cores against the fp32 kernel on the same (bf16-rounded)
     inputs: a prompt portion that continues a context, a whole prompt and two decode rows in one
     step, over shuffled pages; sizes that need padding to the MFMA shapes included."""
@@ -303,6 +321,8 @@ def test_matrix_core_attention_matches_fp32(H, R, dr):
     g = torch.Generator().manual_seed(H * 1000 + R)
     # (context before the run, run length): decodes first, then the portions
     runs = [(130, 1), (63, 1), (70, 37), (0, 90)]
+    if decode_only:  # long contexts, one token each: the keys are cut into ranges and merged
+        runs = [(700, 1), (300, 1), (63, 1), (1500, 1), (0, 1)]
     nblk = [-(-(c + n) // bs) for c, n in runs]
     perm = torch.randperm(sum(nblk) + 2, generator=g)
     tables = torch.zeros(len(runs), max(nblk), dtype=torch.int32)
@@ -316,10 +336,10 @@ def test_matrix_core_attention_matches_fp32(H, R, dr):
     row_seq = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, (_, n) in enumerate(runs)])
     row_len = torch.cat([torch.arange(c + 1, c + n + 1, dtype=torch.int32) for c, n in runs])
     start = torch.tensor([0] + list(torch.tensor([n for _, n in runs]).cumsum(0)), dtype=torch.int32)
-    seq = SeqMeta(num_seqs=len(runs), seq_start=start.to(dev), seq_slot=torch.zeros(4, dtype=torch.int32, device=dev),
-                  seq_init=torch.zeros(4, dtype=torch.int32, device=dev), row_seq=row_seq.to(dev),
-                  row_len=row_len.to(dev), tables=tables.to(dev), max_len=int(row_len.max()), max_q=90,
-                  q_lens=[n for _, n in runs])
+    nz = torch.zeros(len(runs), dtype=torch.int32, device=dev)
+    seq = SeqMeta(num_seqs=len(runs), seq_start=start.to(dev), seq_slot=nz, seq_init=nz, row_seq=row_seq.to(dev),
+                  row_len=row_len.to(dev), tables=tables.to(dev), max_len=int(row_len.max()),
+                  max_q=max(n for _, n in runs), q_lens=[n for _, n in runs])
     scale = Dk ** -0.5
     fast = sm.latent_attention(q.to(dev), cache.to(dev), seq.tables, seq.row_seq, seq.row_len, scale, R, 4, seq=seq)
     slow = sm.latent_attention(q.float().to(dev), cache.float().to(dev), seq.tables, seq.row_seq, seq.row_len, scale, R, 4)
