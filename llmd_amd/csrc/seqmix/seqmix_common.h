@@ -41,6 +41,25 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return s;
 }
 
+// fp32 transcendentals for the sequential scans. float32 storage: the precise library functions.
+// bfloat16 storage: the hardware exp2 / log2 / reciprocal forms (about 1 ulp of fp32, far below the
+// rounding of the values they are applied to); on a single wave per SIMD the precise forms are most
+// of a token's latency.
+template <typename T> struct Fn {
+  static __device__ __forceinline__ float exp(float x) { return expf(x); }
+  static __device__ __forceinline__ float sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
+  static __device__ __forceinline__ float silu(float x) { return x / (1.f + expf(-x)); }
+  static __device__ __forceinline__ float softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+  static __device__ __forceinline__ float rsqrt(float x) { return 1.f / sqrtf(x); }
+};
+template <> struct Fn<uint16_t> {
+  static __device__ __forceinline__ float exp(float x) { return __expf(x); }
+  static __device__ __forceinline__ float sigmoid(float x) { return __frcp_rn(1.f + __expf(-x)); }
+  static __device__ __forceinline__ float silu(float x) { return x * __frcp_rn(1.f + __expf(-x)); }
+  static __device__ __forceinline__ float softplus(float x) { return x > 20.f ? x : __logf(1.f + __expf(x)); }
+  static __device__ __forceinline__ float rsqrt(float x) { return __frsqrt_rn(x); }
+};
+
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float siluf_(float x) { return x / (1.f + expf(-x)); }
 __device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }

@@ -89,42 +89,59 @@ __global__ __launch_bounds__(NT) void selective_scan_kernel(
     S[i] = (n < N && seq_init[s]) ? sp[n] : 0.f;
   }
   const float bias = ld(dt_bias + cc), Dc = ld(D + cc);
-  // inputs are fetched one token ahead of the recurrence
-  float ndt = 0.f, nx = 0.f, nz = 0.f, nB[SPL], nC[SPL];
-  auto fetch = [&](int t) {
-    if (t >= hi) return;
-    ndt = ld(dt_raw + (int64_t)t * C + cc);
-    nx = ld(xc + (int64_t)t * C + cc);
-    nz = ld(xz + (int64_t)t * xz_stride + C + cc);
-    const T* bt = bc + (int64_t)t * bc_stride + R;
+  // inputs are fetched a block of TB tokens ahead of the recurrence: the loads of the next block
+  // are in flight while this block's tokens run one after the other (memory latency is about one
+  // token's worth of arithmetic, a single wave per SIMD cannot hide it otherwise)
+  constexpr int TB = SPL <= 2 ? 8 : 4;
+  float ndt[TB], nx[TB], nz[TB], nB[TB][SPL], nC[TB][SPL];
+  auto fetch = [&](int t0) {
 #pragma unroll
-    for (int i = 0; i < SPL; ++i) {
-      const int n = nl + i * NL;
-      nB[i] = n < N ? ld(bt + n) : 0.f;
-      nC[i] = n < N ? ld(bt + N + n) : 0.f;
-    }
-  };
-  fetch(lo);
-  for (int t = lo; t < hi; ++t) {
-    const float dt = softplusf_(ndt + bias), x = nx, z = nz;
-    float Bv[SPL], Cv[SPL];
+    for (int b = 0; b < TB; ++b) {
+      const int t = min(t0 + b, hi - 1);  // past the end: a valid row, never used
+      ndt[b] = ld(dt_raw + (int64_t)t * C + cc);
+      nx[b] = ld(xc + (int64_t)t * C + cc);
+      nz[b] = ld(xz + (int64_t)t * xz_stride + C + cc);
+      const T* bt = bc + (int64_t)t * bc_stride + R;
 #pragma unroll
-    for (int i = 0; i < SPL; ++i) {
-      Bv[i] = nB[i];
-      Cv[i] = nC[i];
-    }
-    fetch(t + 1);
-    float part = 0.f;
-#pragma unroll
-    for (int i = 0; i < SPL; ++i) {
-      const int n = nl + i * NL;
-      if (n < N) {
-        S[i] = expf(dt * Ac[i]) * S[i] + dt * x * Bv[i];
-        part += S[i] * Cv[i];
+      for (int i = 0; i < SPL; ++i) {
+        const int n = nl + i * NL;
+        nB[b][i] = n < N ? ld(bt + n) : 0.f;
+        nC[b][i] = n < N ? ld(bt + N + n) : 0.f;
       }
     }
-    for (int o = NL >> 1; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
-    if (ok && nl == 0) st(out + (int64_t)t * C + c, (part + Dc * x) * siluf_(z));
+  };
+  if (lo < hi) fetch(lo);
+  for (int t0 = lo; t0 < hi; t0 += TB) {
+    float cdt[TB], cx[TB], cz[TB], cB[TB][SPL], cC[TB][SPL];
+#pragma unroll
+    for (int b = 0; b < TB; ++b) {
+      cdt[b] = ndt[b];
+      cx[b] = nx[b];
+      cz[b] = nz[b];
+#pragma unroll
+      for (int i = 0; i < SPL; ++i) {
+        cB[b][i] = nB[b][i];
+        cC[b][i] = nC[b][i];
+      }
+    }
+    if (t0 + TB < hi) fetch(t0 + TB);
+#pragma unroll
+    for (int b = 0; b < TB; ++b) {
+      const int t = t0 + b;
+      if (t >= hi) break;
+      const float dt = Fn<T>::softplus(cdt[b] + bias), x = cx[b];
+      float part = 0.f;
+#pragma unroll
+      for (int i = 0; i < SPL; ++i) {
+        const int n = nl + i * NL;
+        if (n < N) {
+          S[i] = Fn<T>::exp(dt * Ac[i]) * S[i] + dt * x * cB[b][i];
+          part += S[i] * cC[b][i];
+        }
+      }
+      for (int o = NL >> 1; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+      if (ok && nl == 0) st(out + (int64_t)t * C + c, (part + Dc * x) * Fn<T>::silu(cz[b]));
+    }
   }
   if (ok) {
 #pragma unroll
@@ -137,90 +154,128 @@ __global__ __launch_bounds__(NT) void selective_scan_kernel(
 
 constexpr float DECAY_K = 0.6065306597126334f;  // exp(-1/2)
 
-// KD >= d key channels per thread column; blockDim = BT (a multiple of 64 >= d).
-template <typename T, int KD, int BT>
-__global__ __launch_bounds__(BT) void gdelta_scan_kernel(
+// CT column threads (a multiple of 64 >= d) x NW key groups = 256 threads. Thread (g, j) keeps the
+// KR = KD / NW key rows [g KR, (g + 1) KR) of column j of S in registers (KD >= d, padded rows stay
+// zero). Per token: group 0 computes the key-side vectors (decay, removal rate x unit key, unit key,
+// key, receptance) in fp32 and broadcasts them through LDS; every group forms its part of u^T S and,
+// after the update, of S^T r, and the parts meet in LDS.
+template <typename T, int KD, int CT, int NW>
+__global__ __launch_bounds__(CT * NW) void gdelta_scan_kernel(
     const T* __restrict__ proj, int64_t p_stride, const T* __restrict__ wl, const T* __restrict__ w0,
     const T* __restrict__ a_b, const T* __restrict__ norm_w, float eps, int H, int d, float* __restrict__ state,
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot, const int* __restrict__ seq_init,
     T* __restrict__ out) {
+  constexpr int BT = CT * NW, KR = KD / NW;
   __shared__ __attribute__((aligned(16))) float sw[KD], sau[KD], su[KD], sk[KD], sr[KD];
+  __shared__ float part[NW][CT];
   __shared__ float red[BT / 64];
   const int h = blockIdx.x, s = blockIdx.y;
-  const int j = threadIdx.x;
+  const int j = threadIdx.x % CT, g = threadIdx.x / CT;
   const bool col = j < d;
+  const bool lead = g == 0 && col;
   const int HD = H * d;
   const int lo = seq_start[s], hi = seq_start[s + 1];
   float* sp = state + ((int64_t)seq_slot[s] * H + h) * d * d;
-  float S[KD];
+  const int i0 = g * KR;
+  float S[KR];
   const bool init = seq_init[s] != 0;
 #pragma unroll
-  for (int i = 0; i < KD; ++i) S[i] = (col && i < d && init) ? sp[(int64_t)i * d + j] : 0.f;
-  for (int i = d + j; i < KD; i += BT) sw[i] = sau[i] = su[i] = sk[i] = sr[i] = 0.f;
+  for (int i = 0; i < KR; ++i) S[i] = (col && i0 + i < d && init) ? sp[(int64_t)(i0 + i) * d + j] : 0.f;
+  for (int i = d + threadIdx.x; i < KD; i += BT) sw[i] = sau[i] = su[i] = sk[i] = sr[i] = 0.f;
   const int e = h * d + (col ? j : 0);
   const float w0e = ld(w0 + e), abe = ld(a_b + e), nwe = ld(norm_w + e);
-  // the token's seven inputs of this column are fetched one token ahead, so their latency
-  // overlaps the previous token's arithmetic and barriers
-  float nk = 0.f, na = 0.f, nwl = 0.f, nr = 0.f, nv = 0.f, ng = 0.f;
-  auto fetch = [&](int t) {
-    if (!col || t >= hi) return;
-    const T* pr = proj + (int64_t)t * p_stride;
-    nr = ld(pr + e);
-    nk = ld(pr + HD + e);
-    nv = ld(pr + 2 * HD + e);
-    ng = ld(pr + 3 * HD + e);
-    na = ld(pr + 4 * HD + e);
-    nwl = ld(wl + (int64_t)t * HD + e);
+  // the inputs of this column are fetched a block of TB tokens ahead, so their latency overlaps the
+  // previous block's arithmetic and barriers
+  constexpr int TB = 4;
+  float nk[TB], na[TB], nwl[TB], nr[TB], nv[TB], ng[TB];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int b = 0; b < TB; ++b) {
+      nk[b] = na[b] = nwl[b] = nr[b] = nv[b] = ng[b] = 0.f;
+      const int t = min(t0 + b, hi - 1);  // past the end: a valid row, never used
+      if (!col) continue;
+      const T* pr = proj + (int64_t)t * p_stride;
+      nv[b] = ld(pr + 2 * HD + e);
+      if (g != 0) continue;
+      nr[b] = ld(pr + e);
+      nk[b] = ld(pr + HD + e);
+      ng[b] = ld(pr + 3 * HD + e);
+      na[b] = ld(pr + 4 * HD + e);
+      nwl[b] = ld(wl + (int64_t)t * HD + e);
+    }
   };
-  fetch(lo);
-  for (int t = lo; t < hi; ++t) {
-    const float kj = nk, aj = na, wlj = nwl, rj = nr, v = nv, gj = ng;
-    fetch(t + 1);
-    const float ksum = block_sum<BT>(kj * kj, red);  // also fences the previous token's LDS reads
-    if (col) {
-      const float u = kj / sqrtf(ksum + 1e-6f);
-      const float a = sigmoidf_(aj + abe);
-      sw[j] = expf(-DECAY_K * sigmoidf_(wlj + w0e));
+  if (lo < hi) fetch(lo);
+  for (int t0 = lo; t0 < hi; t0 += TB) {
+    float ck[TB], ca[TB], cwl[TB], cr_[TB], cv[TB], cg[TB];
+#pragma unroll
+    for (int b = 0; b < TB; ++b) {
+      ck[b] = nk[b];
+      ca[b] = na[b];
+      cwl[b] = nwl[b];
+      cr_[b] = nr[b];
+      cv[b] = nv[b];
+      cg[b] = ng[b];
+    }
+    if (t0 + TB < hi) fetch(t0 + TB);
+#pragma unroll
+    for (int b = 0; b < TB; ++b) {
+    const int t = t0 + b;
+    if (t >= hi) break;
+    const float kj = ck[b], aj = ca[b], wlj = cwl[b], rj = cr_[b], v = cv[b], gj = cg[b];
+    const float ksum = block_sum<BT>(lead ? kj * kj : 0.f, red);  // also fences the previous token's LDS reads
+    if (lead) {
+      const float u = kj * Fn<T>::rsqrt(ksum + 1e-6f);
+      const float a = Fn<T>::sigmoid(aj + abe);
+      sw[j] = Fn<T>::exp(-DECAY_K * Fn<T>::sigmoid(wlj + w0e));
       sau[j] = a * u;
       su[j] = u;
       sk[j] = kj;
       sr[j] = rj;
     }
     __syncthreads();
-    float o = 0.f;
-    if (col) {
-      // the key-side vectors come as 16-byte LDS broadcasts; entries beyond d are zero
-      // (written below), so whole groups of four need no bound
-      float sa = 0.f;
+    // the key-side vectors come as 16-byte LDS broadcasts; entries beyond d are zero
+    float sa = 0.f;
 #pragma unroll
-      for (int i = 0; i < KD; i += 4) {
-        if (i < d) {
-          const float4 u4 = *reinterpret_cast<const float4*>(&su[i]);
-          sa += u4.x * S[i] + u4.y * S[i + 1] + u4.z * S[i + 2] + u4.w * S[i + 3];
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < KD; i += 4) {
-        if (i < d) {
-          const float4 w4 = *reinterpret_cast<const float4*>(&sw[i]);
-          const float4 a4 = *reinterpret_cast<const float4*>(&sau[i]);
-          const float4 k4 = *reinterpret_cast<const float4*>(&sk[i]);
-          const float4 r4 = *reinterpret_cast<const float4*>(&sr[i]);
-          S[i] = w4.x * S[i] - a4.x * sa + k4.x * v;
-          S[i + 1] = w4.y * S[i + 1] - a4.y * sa + k4.y * v;
-          S[i + 2] = w4.z * S[i + 2] - a4.z * sa + k4.z * v;
-          S[i + 3] = w4.w * S[i + 3] - a4.w * sa + k4.w * v;
-          o += S[i] * r4.x + S[i + 1] * r4.y + S[i + 2] * r4.z + S[i + 3] * r4.w;
-        }
-      }
+    for (int i = 0; i < KR; i += 4) {
+      const float4 u4 = *reinterpret_cast<const float4*>(&su[i0 + i]);
+      sa += u4.x * S[i] + u4.y * S[i + 1] + u4.z * S[i + 2] + u4.w * S[i + 3];
     }
-    const float ss = block_sum<BT>(o * o, red);
-    if (col) st(out + (int64_t)t * HD + e, o / sqrtf(ss / (float)d + eps) * nwe * sigmoidf_(gj));
+    if (NW > 1) {
+      part[g][j] = sa;
+      __syncthreads();
+      sa = 0.f;
+#pragma unroll
+      for (int q = 0; q < NW; ++q) sa += part[q][j];
+      __syncthreads();
+    }
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < KR; i += 4) {
+      const float4 w4 = *reinterpret_cast<const float4*>(&sw[i0 + i]);
+      const float4 a4 = *reinterpret_cast<const float4*>(&sau[i0 + i]);
+      const float4 k4 = *reinterpret_cast<const float4*>(&sk[i0 + i]);
+      const float4 r4 = *reinterpret_cast<const float4*>(&sr[i0 + i]);
+      S[i] = w4.x * S[i] - a4.x * sa + k4.x * v;
+      S[i + 1] = w4.y * S[i + 1] - a4.y * sa + k4.y * v;
+      S[i + 2] = w4.z * S[i + 2] - a4.z * sa + k4.z * v;
+      S[i + 3] = w4.w * S[i + 3] - a4.w * sa + k4.w * v;
+      o += S[i] * r4.x + S[i + 1] * r4.y + S[i + 2] * r4.z + S[i + 3] * r4.w;
+    }
+    if (NW > 1) {
+      part[g][j] = o;
+      __syncthreads();
+      o = 0.f;
+#pragma unroll
+      for (int q = 0; q < NW; ++q) o += part[q][j];
+    }
+    const float ss = block_sum<BT>(lead ? o * o : 0.f, red);
+    if (lead) st(out + (int64_t)t * HD + e, o * Fn<T>::rsqrt(ss / (float)d + eps) * nwe * Fn<T>::sigmoid(gj));
+    }
   }
   if (col) {
 #pragma unroll
-    for (int i = 0; i < KD; ++i)
-      if (i < d) sp[(int64_t)i * d + j] = S[i];
+    for (int i = 0; i < KR; ++i)
+      if (i0 + i < d) sp[(int64_t)(i0 + i) * d + j] = S[i];
   }
 }
 
@@ -285,21 +340,21 @@ int sm_gdelta_scan(const void* proj, int64_t p_stride, const void* wl, const voi
                    const int* seq_slot, const int* seq_init, void* out, int nseq, int f32, hipStream_t stream) {
   if (nseq == 0) return 0;
   const dim3 grid(H, nseq);
-#define SM_GO(TYPE, KD, BT)                                                                                       \
-  hipLaunchKernelGGL((gdelta_scan_kernel<TYPE, KD, BT>), grid, dim3(BT), 0, stream, (const TYPE*)proj, p_stride,  \
-                     (const TYPE*)wl, (const TYPE*)w0, (const TYPE*)a_b, (const TYPE*)norm_w, eps, H, d, state,   \
-                     seq_start, seq_slot, seq_init, (TYPE*)out)
+#define SM_GO(TYPE, KD, CT, NW)                                                                                  \
+  hipLaunchKernelGGL((gdelta_scan_kernel<TYPE, KD, CT, NW>), grid, dim3(CT * NW), 0, stream, (const TYPE*)proj,   \
+                     p_stride, (const TYPE*)wl, (const TYPE*)w0, (const TYPE*)a_b, (const TYPE*)norm_w, eps, H, d, \
+                     state, seq_start, seq_slot, seq_init, (TYPE*)out)
   if (f32) {
-    if (d <= 32) SM_GO(float, 32, 64);
-    else if (d <= 64) SM_GO(float, 64, 64);
-    else if (d <= 128) SM_GO(float, 128, 128);
-    else if (d <= 256) SM_GO(float, 256, 256);
+    if (d <= 32) SM_GO(float, 32, 64, 4);
+    else if (d <= 64) SM_GO(float, 64, 64, 4);
+    else if (d <= 128) SM_GO(float, 128, 128, 2);
+    else if (d <= 256) SM_GO(float, 256, 256, 1);
     else return 1;
   } else {
-    if (d <= 32) SM_GO(bf16_t, 32, 64);
-    else if (d <= 64) SM_GO(bf16_t, 64, 64);
-    else if (d <= 128) SM_GO(bf16_t, 128, 128);
-    else if (d <= 256) SM_GO(bf16_t, 256, 256);
+    if (d <= 32) SM_GO(bf16_t, 32, 64, 4);
+    else if (d <= 64) SM_GO(bf16_t, 64, 64, 4);
+    else if (d <= 128) SM_GO(bf16_t, 128, 128, 2);
+    else if (d <= 256) SM_GO(bf16_t, 256, 256, 1);
     else return 1;
   }
 #undef SM_GO
