@@ -236,54 +236,34 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
   const int nsplit = gridDim.y;
   const int kbeg = nsplit > 1 ? blockIdx.y * split_keys : 0;
   const int kend = nsplit > 1 ? min(maxlen, kbeg + split_keys) : maxlen;
-  // A tile's chunks (8 bf16 each) are fetched into registers all at once, one tile ahead of the
-  // MFMAs that use it, and go to LDS at the top of the next iteration: the global-memory latency
-  // is paid once per tile and overlaps the previous tile's arithmetic.
-  constexpr int CPR = DkP / 8;                       // chunks per key row
-  constexpr int NCH = (MKT * CPR + NT - 1) / NT;     // chunks per thread
-  u32x4_t pre[NCH];
-  auto gload = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int e = threadIdx.x + i * NT;
-      const int j = e / CPR, c = e - j * CPR;
+  for (int k0 = kbeg; k0 < kend; k0 += MKT) {
+    __syncthreads();  // the previous tile is no longer read
+    // consecutive lanes take consecutive keys of one 8-column chunk: the transposed 2-byte writes
+    // below then fall into consecutive LDS words (chunk-major lanes would all hit one bank)
+    for (int e = threadIdx.x; e < MKT * (DkP / 8); e += NT) {
+      const int c = e / MKT, j = e - c * MKT;
       const int key = k0 + j;
-      __attribute__((aligned(16))) bf16_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (e < MKT * CPR && key < kend && c * 8 < Dk) {
+      __attribute__((aligned(16))) bf16_t v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = 0;
+      if (key < kend) {
         const bf16_t* src = cache + ((int64_t)bt[key / bs] * bs + (key % bs)) * Dk + c * 8;
         if (vec && c * 8 + 8 <= Dk) {
           *reinterpret_cast<u32x4_t*>(v) = *reinterpret_cast<const u32x4_t*>(src);
         } else {
 #pragma unroll
-          for (int q = 0; q < 8; ++q)
-            if (c * 8 + q < Dk) v[q] = src[q];
+          for (int i = 0; i < 8; ++i)
+            if (c * 8 + i < Dk) v[i] = src[i];
         }
       }
-      pre[i] = *reinterpret_cast<u32x4_t*>(v);
-    }
-  };
-  auto lstore = [&]() {
+      *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = *reinterpret_cast<u32x4_t*>(v);
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int e = threadIdx.x + i * NT;
-      if (e >= MKT * CPR) continue;
-      const int j = e / CPR, c = e - j * CPR;
-      *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = pre[i];
-      __attribute__((aligned(16))) bf16_t v[8];
-      *reinterpret_cast<u32x4_t*>(v) = pre[i];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const int d = c * 8 + q;
-        if (d < RP) sVt[d * VS + j] = d < R ? v[q] : (bf16_t)0;
+      for (int i = 0; i < 8; ++i) {
+        const int d = c * 8 + i;
+        if (d < RP) sVt[d * VS + j] = d < R ? v[i] : (bf16_t)0;
       }
     }
-  };
-  if (kbeg < kend) gload(kbeg);
-  for (int k0 = kbeg; k0 < kend; k0 += MKT) {
-    __syncthreads();  // the previous tile is no longer read
-    lstore();
     __syncthreads();
-    if (k0 + MKT < kend) gload(k0 + MKT);
     // scores of this lane's row against keys k0 + 16 kb + 4 kq + r
     float sc[2][4];
 #pragma unroll
