@@ -30,7 +30,7 @@ int sm_gdelta_scan(const void*, int64_t, const void*, const void*, const void*, 
                    const int*, const int*, const int*, void*, int, int, hipStream_t);
 void sm_moe_route(const float*, int, int, int*, float*, int, hipStream_t);
 void sm_moe_group(const int*, int, int, int*, int*, int*, int, hipStream_t);
-void sm_moe_gemm(const void*, int64_t, int, const int*, const int*, const void*, int, int, void*, int, int, int,
+void sm_moe_gemm(const void*, int64_t, int, const int*, const int*, const void*, int, int, void*, int, int, int, int,
                  hipStream_t);
 void sm_moe_combine(const void*, const int*, const float*, int, int, void*, int, int, hipStream_t);
 }
@@ -310,7 +310,7 @@ void moe_group(Tensor ids, int64_t E, Tensor slot_row, Tensor tile_e, Tensor pai
                mt, cur());
 }
 
-void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, Tensor C, bool gelu) {
+void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, Tensor C, bool gelu, int64_t rows) {
   const c10::hip::OptionalHIPGuard g(dev_of(A));
   TORCH_CHECK(A.is_cuda() && act_ok(A) && A.dim() == 2 && A.stride(1) == 1, "A");
   CHECK_ACT(W, A);
@@ -323,7 +323,7 @@ void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, 
                   C.size(1) == W.size(1), "C [tiles * 64, N]");
   TORCH_CHECK(kdiv > 0 || A.size(0) == mt * 64, "A rows are the tile slots");
   sm_moe_gemm(A.data_ptr(), A.stride(0), kdiv, slot_row.data_ptr<int>(), tile_e.data_ptr<int>(), W.data_ptr(),
-              W.size(1), W.size(2), C.data_ptr(), mt, gelu ? 1 : 0, is_f32(A), cur());
+              W.size(1), W.size(2), C.data_ptr(), mt, rows, gelu ? 1 : 0, is_f32(A), cur());
 }
 
 void moe_combine(Tensor y, Tensor pair_slot, Tensor w, Tensor out) {

@@ -201,9 +201,12 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-constexpr int MBN = 128, MBK = 64, MLS = MBK + 8;  // LDS row stride 144 B
+constexpr int MBK = 64, MLS = MBK + 8;  // LDS row stride 144 B
 
-template <bool GELU>
+// NJ = 16-column fragments per wave: the workgroup's tile is 64 rows x MBN = 32 NJ columns
+// (128 for steps with few rows per expert: more workgroups stream the weights; 256 for prompt-sized
+// steps: twice the MFMAs per LDS pass and barrier).
+template <bool GELU, int NJ>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __restrict__ A, int64_t a_stride, int kdiv,
                                                             const int* __restrict__ slot_row,
                                                             const int* __restrict__ tile_e,
@@ -211,6 +214,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
                                                             bf16_t* __restrict__ Cout) {
   const int e = tile_e[blockIdx.x];
   if (e < 0) return;
+  constexpr int MBN = 32 * NJ, NB = MBN / 32;  // NB = B chunks per thread and K step
   __shared__ __attribute__((aligned(16))) bf16_t sA[TM * MLS];
   __shared__ __attribute__((aligned(16))) bf16_t sB[MBN * MLS];
   __shared__ int srow[TM];
@@ -223,8 +227,8 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
   }
   __syncthreads();
   const bf16_t* We = Wt + (int64_t)e * N * K;
-  // staging: A 64 rows x 8 chunks of 16 B (2 per thread), B 128 x 8 (4 per thread)
-  u32x4_t ra[2], rb[4];
+  // staging: A 64 rows x 8 chunks of 16 B (2 per thread), B MBN x 8 (NB per thread)
+  u32x4_t ra[2], rb[NB];
   auto load = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -235,7 +239,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
       ra[i] = v;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const int c = tid + 256 * i, r = c >> 3, ch = c & 7;
       u32x4_t v = {0, 0, 0, 0};
       if (n0 + r < N && k0 + ch * 8 < K) v = *reinterpret_cast<const u32x4_t*>(We + (int64_t)(n0 + r) * K + k0 + ch * 8);
@@ -249,16 +253,16 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
       *reinterpret_cast<u32x4_t*>(&sA[(c >> 3) * MLS + (c & 7) * 8]) = ra[i];
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const int c = tid + 256 * i;
       *reinterpret_cast<u32x4_t*>(&sB[(c >> 3) * MLS + (c & 7) * 8]) = rb[i];
     }
   };
-  f32x4_t acc[2][4];
+  f32x4_t acc[2][NJ];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NJ; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const int r16 = lane & 15, kq = lane >> 4;
   const int nk = (K + MBK - 1) / MBK;
   load(0);
@@ -269,20 +273,20 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
     if (kt + 1 < nk) load((kt + 1) * MBK);
 #pragma unroll
     for (int ks = 0; ks < MBK / 32; ++ks) {
-      bf16x8_t af[2], bfr[4];
+      bf16x8_t af[2], bfr[NJ];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
         af[i] = *reinterpret_cast<const bf16x8_t*>(&sA[(wm * 32 + i * 16 + r16) * MLS + ks * 32 + kq * 8]);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        bfr[j] = *reinterpret_cast<const bf16x8_t*>(&sB[(wn * 64 + j * 16 + r16) * MLS + ks * 32 + kq * 8]);
+      for (int j = 0; j < NJ; ++j)
+        bfr[j] = *reinterpret_cast<const bf16x8_t*>(&sB[(wn * 16 * NJ + j * 16 + r16) * MLS + ks * 32 + kq * 8]);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
     }
   }
-  // acc[i][j][r] = C[row 32 wm + 16 i + 4 kq + r][column 64 wn + 16 j + r16]
+  // acc[i][j][r] = C[row 32 wm + 16 i + 4 kq + r][column 16 NJ wn + 16 j + r16]
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -290,8 +294,8 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
       const int row = wm * 32 + i * 16 + kq * 4 + r;
       if (srow[row] < 0) continue;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int n = n0 + wn * 64 + j * 16 + r16;
+      for (int j = 0; j < NJ; ++j) {
+        const int n = n0 + wn * 16 * NJ + j * 16 + r16;
         if (n >= N) continue;
         float v = acc[i][j][r];
         if (GELU) v = 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
@@ -332,15 +336,23 @@ void sm_moe_group(const int* ids, int n, int E, int* slot_row, int* tile_e, int*
 }
 
 void sm_moe_gemm(const void* A, int64_t a_stride, int kdiv, const int* slot_row, const int* tile_e, const void* W,
-                 int N, int K, void* C, int max_tiles, int gelu, int f32, hipStream_t stream) {
+                 int N, int K, void* C, int max_tiles, int rows_hint, int gelu, int f32, hipStream_t stream) {
   if (!f32 && K % 8 == 0 && a_stride % 8 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0) {
-    const dim3 g2(max_tiles, (N + MBN - 1) / MBN);
-    if (gelu)
-      hipLaunchKernelGGL((moe_gemm_mfma_kernel<true>), g2, dim3(256), 0, stream, (const bf16_t*)A, a_stride, kdiv,
-                         slot_row, tile_e, (const bf16_t*)W, N, K, (bf16_t*)C);
-    else
-      hipLaunchKernelGGL((moe_gemm_mfma_kernel<false>), g2, dim3(256), 0, stream, (const bf16_t*)A, a_stride, kdiv,
-                         slot_row, tile_e, (const bf16_t*)W, N, K, (bf16_t*)C);
+    // wide tiles when the step has prompt-sized row counts (most tiles are full) and N is wide
+    const bool wide = N >= 256 && rows_hint >= 32 * max_tiles;
+    const int mbn = wide ? 256 : 128;
+    const dim3 g2(max_tiles, (N + mbn - 1) / mbn);
+#define SM_MF(G, NJ)                                                                                          \
+  hipLaunchKernelGGL((moe_gemm_mfma_kernel<G, NJ>), g2, dim3(256), 0, stream, (const bf16_t*)A, a_stride, kdiv, \
+                     slot_row, tile_e, (const bf16_t*)W, N, K, (bf16_t*)C)
+    if (gelu) {
+      if (wide) SM_MF(true, 8);
+      else SM_MF(true, 4);
+    } else {
+      if (wide) SM_MF(false, 8);
+      else SM_MF(false, 4);
+    }
+#undef SM_MF
     return;
   }
   const dim3 grid(max_tiles, (N + TN - 1) / TN);

@@ -197,8 +197,8 @@ def moe_ffn(h, ids, w, w1, w2):
     C.moe_group(ids, E, slot_row, tile_e, pair_slot)
     a = torch.empty(max_tiles * MOE_TILE, Fh, dtype=h.dtype, device=dev)
     y = torch.empty(max_tiles * MOE_TILE, d, dtype=h.dtype, device=dev)
-    C.moe_gemm(h, k, slot_row, tile_e, w1, a, True)
-    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, False)
+    C.moe_gemm(h, k, slot_row, tile_e, w1, a, True, n)   # n = rows of the step: picks the tile width
+    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, False, n)
     out = torch.empty_like(h)
     C.moe_combine(y, pair_slot, w, out)
     return out

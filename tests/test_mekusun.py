@@ -349,7 +349,8 @@ def test_matrix_core_attention_matches_fp32(H, R, dr, decode_only):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("T,d,F,E,k", [(70, 48, 24, 5, 2), (300, 256, 200, 16, 3), (9, 64, 72, 4, 4), (33, 50, 30, 3, 1)])
+@pytest.mark.parametrize("T,d,F,E,k", [(70, 48, 24, 5, 2), (300, 256, 200, 16, 3), (9, 64, 72, 4, 4), (33, 50, 30, 3, 1),
+                                       (1500, 256, 328, 4, 2)])  # the last: prompt-sized, the wide tiles
 def test_expert_gemm_bf16_matches_fp32(T, d, F, E, k):
     """The bfloat16 expert feed-forward (matrix cores where rows are 16-byte aligned, the FMA
     kernel otherwise) against the float32 kernels on the same bf16-rounded inputs."""
