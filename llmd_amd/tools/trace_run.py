@@ -3,7 +3,9 @@
     bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
 
 Standard input: one JSON object per line,
-    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+    {"step": 7, "entries": [{"id": "r1", "tokens": [11, 4, 90, 2], "want": [3]}, {"id": "r2", "tokens": [8], "want": []}],
+     "end": ["r2"]}
+(on one line)
 ``entries`` bring each request's next tokens (a request is admitted at its first entry and may
 skip steps); ``want`` are the places among them whose logits are written; ``end`` lists the
 requests finished after the step. All entries of a step run as one batch of the engine's own

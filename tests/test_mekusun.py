@@ -373,3 +373,34 @@ def test_expert_gemm_bf16_matches_fp32(T, d, F, E, k):
             want[t] += float(w[t, j]) * (oracle.gelu_erf(h[t].double() @ w1[e].double().T) @ w2[e].double().T)
     assert float((slow.cpu().double() - want).abs().max() / want.abs().max()) < 1e-5
     assert float((fast.float() - slow).abs().max() / slow.abs().max()) < 2e-2
+
+
+def test_trace_runner_program(tmp_path):
+    """bin/trace_run as a program: steps on standard input, 'done <step>' lines, one fp32 file per step
+    with wanted places; a request that skips a step, ends, and a later one that reuses its slot."""
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    path, W = model_dir(tmp_path, NO_ATTENTION, seed=3)
+    a, b, c = (tokens(n, NO_ATTENTION["vocab"], 40 + i) for i, n in enumerate((9, 3, 5)))
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:6], "want": [0, 5]}, {"id": "b", "tokens": b[:2], "want": []}],
+              "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[6:7], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[2:], "want": [0]}, {"id": "a", "tokens": a[7:], "want": [1]}],
+              "end": ["a", "b"]},
+             {"step": 3, "entries": [{"id": "c", "tokens": c, "want": [4]}], "end": ["c"]}]
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128", "--max-seqs", "2", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    V = NO_ATTENTION["vocab"]
+    la, lb, lc = (oracle.forward(NO_ATTENTION, W, t) for t in (a, b, c))
+    want = {0: torch.stack([la[0], la[5]]), 1: la[6:7], 2: torch.stack([lb[2], la[8]]), 3: lc[4:5]}
+    for i, w in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V).copy())
+        assert got.shape == w.shape and rel_err(got, w) < TOL["float32"], i
