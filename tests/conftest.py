@@ -44,3 +44,11 @@ def _seed_torch():
 
     torch.manual_seed(int(os.environ.get("LLMD_TEST_SEED", "0")))
     yield
+
+
+def skip_if_vmm_import_refused(text: str):
+    """A box may refuse to import another process's shareable VMM handle on the SAME GPU
+    (hipMemImportFromShareableHandle -> invalid value: 'vmm import failed: 1'), e.g. for an
+    unprivileged user. Tests of that path skip there; everything else they assert still holds."""
+    if "vmm import failed" in text:
+        pytest.skip("this box refuses cross-process VMM handle imports on one GPU (vmm import failed)")

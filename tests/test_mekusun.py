@@ -198,13 +198,15 @@ def test_mixed_batches_reuse_pages_and_slots(tmp_path, device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("cfg", [PLAIN, NO_ATTENTION], ids=["equal-or-one", "no-attention"])
-def test_other_sizes(tmp_path, device, cfg):
+def test_other_sizes(tmp_path, device, cfg, dtype):
     path, W = model_dir(tmp_path, cfg, seed=5)
     toks = tokens(80, cfg["vocab"], 6)
     want = oracle.forward(cfg, W, toks)
-    got = replay(engine(path, device), {"a": toks}, [[("a", 5)], [("a", 60)], [("a", 2)]] + [[("a", 1)]] * 13)["a"]
-    assert rel_err(got, want) < TOL["float32"]
+    got = replay(engine(path, device, dtype), {"a": toks},
+                 [[("a", 5)], [("a", 60)], [("a", 2)]] + [[("a", 1)]] * 13)["a"]
+    assert rel_err(got, want) < TOL[dtype]
 
 
 def _paged(keys, block_size, device, dtype):
