@@ -60,8 +60,6 @@ template <> struct Fn<uint16_t> {
   static __device__ __forceinline__ float rsqrt(float x) { return __frsqrt_rn(x); }
 };
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float siluf_(float x) { return x / (1.f + expf(-x)); }
-__device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
 }  // namespace sm

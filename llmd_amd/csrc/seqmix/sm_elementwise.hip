@@ -103,12 +103,6 @@ __global__ __launch_bounds__(NT) void softcap_kernel(float* __restrict__ x, floa
 
 }  // namespace
 
-#define SM_DISPATCH(f32, KERNEL, grid, ...)                                             \
-  do {                                                                                   \
-    if (f32) hipLaunchKernelGGL((KERNEL<float>), grid, dim3(NT), 0, stream, __VA_ARGS__); \
-    else hipLaunchKernelGGL((KERNEL<bf16_t>), grid, dim3(NT), 0, stream, __VA_ARGS__);    \
-  } while (0)
-
 extern "C" {
 
 void sm_embed_scale(const int64_t* ids, const void* table, float scale, float* o0, float* o1, int T, int d,

@@ -219,57 +219,57 @@ __global__ __launch_bounds__(CT * NW) void gdelta_scan_kernel(
     if (t0 + TB < hi) fetch(t0 + TB);
 #pragma unroll
     for (int b = 0; b < TB; ++b) {
-    const int t = t0 + b;
-    if (t >= hi) break;
-    const float kj = ck[b], aj = ca[b], wlj = cwl[b], rj = cr_[b], v = cv[b], gj = cg[b];
-    const float ksum = block_sum<BT>(lead ? kj * kj : 0.f, red);  // also fences the previous token's LDS reads
-    if (lead) {
-      const float u = kj * Fn<T>::rsqrt(ksum + 1e-6f);
-      const float a = Fn<T>::sigmoid(aj + abe);
-      sw[j] = Fn<T>::exp(-DECAY_K * Fn<T>::sigmoid(wlj + w0e));
-      sau[j] = a * u;
-      su[j] = u;
-      sk[j] = kj;
-      sr[j] = rj;
-    }
-    __syncthreads();
-    // the key-side vectors come as 16-byte LDS broadcasts; entries beyond d are zero
-    float sa = 0.f;
-#pragma unroll
-    for (int i = 0; i < KR; i += 4) {
-      const float4 u4 = *reinterpret_cast<const float4*>(&su[i0 + i]);
-      sa += u4.x * S[i] + u4.y * S[i + 1] + u4.z * S[i + 2] + u4.w * S[i + 3];
-    }
-    if (NW > 1) {
-      part[g][j] = sa;
+      const int t = t0 + b;
+      if (t >= hi) break;
+      const float kj = ck[b], aj = ca[b], wlj = cwl[b], rj = cr_[b], v = cv[b], gj = cg[b];
+      const float ksum = block_sum<BT>(lead ? kj * kj : 0.f, red);  // also fences the previous token's LDS reads
+      if (lead) {
+        const float u = kj * Fn<T>::rsqrt(ksum + 1e-6f);
+        const float a = Fn<T>::sigmoid(aj + abe);
+        sw[j] = Fn<T>::exp(-DECAY_K * Fn<T>::sigmoid(wlj + w0e));
+        sau[j] = a * u;
+        su[j] = u;
+        sk[j] = kj;
+        sr[j] = rj;
+      }
       __syncthreads();
-      sa = 0.f;
+      // the key-side vectors come as 16-byte LDS broadcasts; entries beyond d are zero
+      float sa = 0.f;
 #pragma unroll
-      for (int q = 0; q < NW; ++q) sa += part[q][j];
-      __syncthreads();
-    }
-    float o = 0.f;
+      for (int i = 0; i < KR; i += 4) {
+        const float4 u4 = *reinterpret_cast<const float4*>(&su[i0 + i]);
+        sa += u4.x * S[i] + u4.y * S[i + 1] + u4.z * S[i + 2] + u4.w * S[i + 3];
+      }
+      if (NW > 1) {
+        part[g][j] = sa;
+        __syncthreads();
+        sa = 0.f;
 #pragma unroll
-    for (int i = 0; i < KR; i += 4) {
-      const float4 w4 = *reinterpret_cast<const float4*>(&sw[i0 + i]);
-      const float4 a4 = *reinterpret_cast<const float4*>(&sau[i0 + i]);
-      const float4 k4 = *reinterpret_cast<const float4*>(&sk[i0 + i]);
-      const float4 r4 = *reinterpret_cast<const float4*>(&sr[i0 + i]);
-      S[i] = w4.x * S[i] - a4.x * sa + k4.x * v;
-      S[i + 1] = w4.y * S[i + 1] - a4.y * sa + k4.y * v;
-      S[i + 2] = w4.z * S[i + 2] - a4.z * sa + k4.z * v;
-      S[i + 3] = w4.w * S[i + 3] - a4.w * sa + k4.w * v;
-      o += S[i] * r4.x + S[i + 1] * r4.y + S[i + 2] * r4.z + S[i + 3] * r4.w;
-    }
-    if (NW > 1) {
-      part[g][j] = o;
-      __syncthreads();
-      o = 0.f;
+        for (int q = 0; q < NW; ++q) sa += part[q][j];
+        __syncthreads();
+      }
+      float o = 0.f;
 #pragma unroll
-      for (int q = 0; q < NW; ++q) o += part[q][j];
-    }
-    const float ss = block_sum<BT>(lead ? o * o : 0.f, red);
-    if (lead) st(out + (int64_t)t * HD + e, o * Fn<T>::rsqrt(ss / (float)d + eps) * nwe * Fn<T>::sigmoid(gj));
+      for (int i = 0; i < KR; i += 4) {
+        const float4 w4 = *reinterpret_cast<const float4*>(&sw[i0 + i]);
+        const float4 a4 = *reinterpret_cast<const float4*>(&sau[i0 + i]);
+        const float4 k4 = *reinterpret_cast<const float4*>(&sk[i0 + i]);
+        const float4 r4 = *reinterpret_cast<const float4*>(&sr[i0 + i]);
+        S[i] = w4.x * S[i] - a4.x * sa + k4.x * v;
+        S[i + 1] = w4.y * S[i + 1] - a4.y * sa + k4.y * v;
+        S[i + 2] = w4.z * S[i + 2] - a4.z * sa + k4.z * v;
+        S[i + 3] = w4.w * S[i + 3] - a4.w * sa + k4.w * v;
+        o += S[i] * r4.x + S[i + 1] * r4.y + S[i + 2] * r4.z + S[i + 3] * r4.w;
+      }
+      if (NW > 1) {
+        part[g][j] = o;
+        __syncthreads();
+        o = 0.f;
+#pragma unroll
+        for (int q = 0; q < NW; ++q) o += part[q][j];
+      }
+      const float ss = block_sum<BT>(lead ? o * o : 0.f, red);
+      if (lead) st(out + (int64_t)t * HD + e, o * Fn<T>::rsqrt(ss / (float)d + eps) * nwe * Fn<T>::sigmoid(gj));
     }
   }
   if (col) {
