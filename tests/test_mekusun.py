@@ -59,6 +59,11 @@ MIXED = config([(attn(3, 24, 8, 16, 40, rot_dims=4, base=500.0), dense(72)),
 PLAIN = config([(mamba(32, 1, 1, 1), None),
                 (attn(1, 16, 16, 16, 16), moe(16, 4, 4)),
                 (delta(1, 64), dense(64))], width=32, vocab=64, scale=1.0, cap=0.0)
+# sizes that are multiples of nothing: vector loads, MFMA padding and lane groups all take their slow paths
+ODD = config([(attn(7, 10, 6, 14, 18, base=77.0), moe(22, 7, 3)),
+              (delta(2, 50), dense(26)),
+              (mamba(30, 3, 2, 5), None),
+              (mamba(20, 100, 7, 2), moe(10, 2, 2))], width=34, vocab=51, scale=0.5, cap=7.0, eps=1e-4)
 NO_ATTENTION = config([(delta(2, 16), dense(40)), (mamba(24, 8, 4, 3), None)], width=24, vocab=40)
 
 
@@ -199,7 +204,7 @@ def test_mixed_batches_reuse_pages_and_slots(tmp_path, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("cfg", [PLAIN, NO_ATTENTION], ids=["equal-or-one", "no-attention"])
+@pytest.mark.parametrize("cfg", [PLAIN, NO_ATTENTION, ODD], ids=["equal-or-one", "no-attention", "odd"])
 def test_other_sizes(tmp_path, device, cfg, dtype):
     path, W = model_dir(tmp_path, cfg, seed=5)
     toks = tokens(80, cfg["vocab"], 6)
