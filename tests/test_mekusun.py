@@ -411,3 +411,20 @@ def test_trace_runner_program(tmp_path):
     for i, w in want.items():
         got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V).copy())
         assert got.shape == w.shape and rel_err(got, w) < TOL["float32"], i
+
+
+@pytest.mark.parametrize("async_sched", [False, True], ids=["sync", "async"])
+def test_preemption_recomputes_state(tmp_path, async_sched):
+    """A pool too small for both requests' growth: one is preempted (pages and state slot freed),
+    recomputed from its first token, and still generates what an unconstrained engine generates."""
+    path, _ = model_dir(tmp_path, MIXED, seed=9)
+    prompts = [tokens(50, MIXED["vocab"], 30), tokens(50, MIXED["vocab"], 31)]
+    sp = SamplingParams(max_tokens=24, temperature=0.0, ignore_eos=True)
+    roomy = engine(path, "cpu", pages=8, seqs=2, async_scheduling=async_sched)
+    want = [r.output_token_ids for r in roomy.generate(prompts, sp)]
+    tight = engine(path, "cpu", pages=2, seqs=2, async_scheduling=async_sched)
+    got = [r.output_token_ids for r in tight.generate(prompts, sp)]
+    assert tight.sched.num_preemptions_total > 0
+    assert got == want
+    tight.bm.check_invariants()
+    assert tight.bm.num_free() == 2 and tight.bm.slots.num_free() == 2
