@@ -199,10 +199,15 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, int split_keys, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int DkP = 32 * NKS, RP = 16 * NCB;
   constexpr int KS = DkP + 8, VS = MKT + 8, PS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
+  // The weights P live in the key tile's space once the scores are done (one more barrier per
+  // tile) when the tile is large enough: the largest form then needs 78 KB of LDS and two
+  // workgroups share a CU, one staging its tile while the other multiplies.
+  constexpr bool ALIAS = MKT * KS >= 2 * 4 * 16 * PS;
   __shared__ __attribute__((aligned(16))) bf16_t sK[MKT * KS];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[RP * VS];
-  __shared__ __attribute__((aligned(16))) bf16_t sPh[4 * 16 * PS];
-  __shared__ __attribute__((aligned(16))) bf16_t sPl[4 * 16 * PS];
+  __shared__ __attribute__((aligned(16))) bf16_t sP[ALIAS ? 8 : 2 * 4 * 16 * PS];
+  bf16_t* const sPh = ALIAS ? sK : sP;
+  bf16_t* const sPl = sPh + 4 * 16 * PS;
   const int seq = items[blockIdx.x * 3], tok0 = items[blockIdx.x * 3 + 1], ntok = items[blockIdx.x * 3 + 2];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, kq = lane >> 4;
@@ -238,29 +243,46 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
   const int kend = nsplit > 1 ? min(maxlen, kbeg + split_keys) : maxlen;
   for (int k0 = kbeg; k0 < kend; k0 += MKT) {
     __syncthreads();  // the previous tile is no longer read
-    // consecutive lanes take consecutive keys of one 8-column chunk: the transposed 2-byte writes
-    // below then fall into consecutive LDS words (chunk-major lanes would all hit one bank)
-    for (int e = threadIdx.x; e < MKT * (DkP / 8); e += NT) {
+    // The tile's 16-byte chunks are all requested before any of them is used: one memory latency
+    // per tile, not one per chunk. A tile lies inside one page when the page size is a multiple of
+    // the tile (tiles start at multiples of 32 keys), so its block-table entry is read once.
+    // Consecutive lanes take consecutive keys of one 8-column chunk: the transposed 2-byte writes
+    // then fall into consecutive LDS words (chunk-major lanes would all hit one bank).
+    constexpr int CPR = DkP / 8;                    // chunks per key row
+    constexpr int NCH = (MKT * CPR + NT - 1) / NT;  // chunks per thread
+    const bool one_page = (bs % MKT) == 0;
+    const int64_t row0 = one_page ? (int64_t)bt[k0 / bs] * bs + (k0 % bs) : 0;
+    u32x4_t pre[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int e = threadIdx.x + i * NT;
       const int c = e / MKT, j = e - c * MKT;
       const int key = k0 + j;
-      __attribute__((aligned(16))) bf16_t v[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = 0;
-      if (key < kend) {
-        const bf16_t* src = cache + ((int64_t)bt[key / bs] * bs + (key % bs)) * Dk + c * 8;
+      u32x4_t v = {0, 0, 0, 0};
+      if (e < MKT * CPR && key < kend && c * 8 < Dk) {
+        const int64_t row = one_page ? row0 + j : (int64_t)bt[key / bs] * bs + (key % bs);
+        const bf16_t* src = cache + row * Dk + c * 8;
         if (vec && c * 8 + 8 <= Dk) {
-          *reinterpret_cast<u32x4_t*>(v) = *reinterpret_cast<const u32x4_t*>(src);
+          v = *reinterpret_cast<const u32x4_t*>(src);
         } else {
 #pragma unroll
-          for (int i = 0; i < 8; ++i)
-            if (c * 8 + i < Dk) v[i] = src[i];
+          for (int q = 0; q < 8; ++q)
+            if (c * 8 + q < Dk) v[q >> 1] |= (uint32_t)src[q] << (16 * (q & 1));
         }
       }
-      *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = *reinterpret_cast<u32x4_t*>(v);
+      pre[i] = v;
+    }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int d = c * 8 + i;
-        if (d < RP) sVt[d * VS + j] = d < R ? v[i] : (bf16_t)0;
+    for (int i = 0; i < NCH; ++i) {
+      const int e = threadIdx.x + i * NT;
+      if (e >= MKT * CPR) continue;
+      const int c = e / MKT, j = e - c * MKT;
+      *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = pre[i];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const int d = c * 8 + q;
+        const bf16_t val = (bf16_t)(pre[i][q >> 1] >> (16 * (q & 1)));
+        if (d < RP) sVt[d * VS + j] = d < R ? val : (bf16_t)0;
       }
     }
     __syncthreads();
@@ -278,6 +300,7 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
       for (int r = 0; r < 4; ++r)
         sc[kb][r] = (k0 + kb * 16 + kq * 4 + r < min(mylen, kend)) ? a[r] * scale : -INFINITY;
     }
+    if (ALIAS) __syncthreads();  // every wave has read its keys: their space takes the weights
     float mx = -INFINITY;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
