@@ -72,6 +72,8 @@ class ModelConfig:
     layer_specs: Optional[list] = None
     embedding_scale: float = 1.0
     logit_softcap: float = 0.0
+    # hyper-connections (models/negunex.py): number of residual streams, 0 = one plain residual
+    hyper_streams: int = 0
     name: str = "custom"
 
     def __post_init__(self):
@@ -117,6 +119,8 @@ class ModelConfig:
                 st = os.path.join(os.path.dirname(p), "model.safetensors")
                 shapes = safetensors_shapes(st) if os.path.exists(st) else {}
             return mekusun_config(d, shapes)
+        if d.get("architecture") == "Negunex":
+            return negunex_config(d)
         names = {f.name for f in dataclasses.fields(cls)}
         kw = {k: v for k, v in d.items() if k in names}
         if "num_experts" in d and "num_local_experts" not in d:
@@ -173,6 +177,31 @@ def mekusun_config(d: dict, shapes: Optional[dict] = None) -> ModelConfig:
         bos_token_id=d.get("bos", 0), eos_token_id=d.get("eos", -1), layer_specs=layers,
         embedding_scale=d.get("embedding", {}).get("scale", 1.0), logit_softcap=d.get("logit_softcap", 0.0),
         name=d.get("name", "mekusun"))
+
+
+def negunex_config(d: dict) -> ModelConfig:
+    """A Negunex ``config.json``: attention layers listed one by one (``layers``: type, ``mixer``
+    sizes and constants, ``mlp`` or null), ``streams`` residual streams joined by hyper-connections,
+    ``norm.eps``, ``vocab``, ``width``. The generic fields the engine reads are filled from the
+    first attention layer; everything per layer stays in ``layer_specs``."""
+    layers = [json.loads(json.dumps(l)) for l in d["layers"]]
+    for i, l in enumerate(layers):
+        if l["type"] != "attention":
+            raise ValueError(f"negunex: layer {i} has the unknown mixer type {l['type']!r}")
+    moe = [l["mlp"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "moe"]
+    att = [l["mixer"] for l in layers]
+    return ModelConfig(
+        model_type="negunex", hidden_size=d["width"], vocab_size=d["vocab"], num_hidden_layers=len(layers),
+        num_attention_heads=att[0]["heads"] if att else 1, num_key_value_heads=att[0]["kv_heads"] if att else 1,
+        head_dim=att[0]["dim"] if att else 1, v_head_dim=att[0]["vdim"] if att else 0,
+        intermediate_size=max([l["mlp"]["ff"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "dense"]
+                              or [0]),
+        num_local_experts=max([m["router"]["experts"] for m in moe] or [0]),
+        num_experts_per_tok=max([m["router"]["top"] for m in moe] or [0]),
+        moe_intermediate_size=max([m["expert"]["ff"] for m in moe] or [0]),
+        rms_norm_eps=d["norm"]["eps"], max_position_embeddings=d.get("max_position", 1 << 20),
+        bos_token_id=d.get("bos", 0), eos_token_id=d.get("eos", -1), layer_specs=layers,
+        hyper_streams=int(d.get("streams") or 0), name=d.get("name", "negunex"))
 
 
 def _llama(name, d, ffn, L, hq, hkv, vocab=128256, **kw):

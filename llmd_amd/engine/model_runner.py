@@ -158,12 +158,15 @@ class ModelRunner:
         # layers with per-sequence recurrent state: slots in engine/state_cache.py; steps are
         # described per sequence (AttnMeta.seq)
         self.stateful = bool(getattr(self.model, "stateful", False))
+        # per-layer stacks without recurrent state use the same per-sequence step description
+        self.seq_steps = self.stateful or bool(getattr(self.model, "seq_steps", False))
         self.state_pool = None
+        if self.seq_steps and (cfg.kv_transfer_config or cfg.kv_offload_config or cfg.enable_lora):
+            raise ValueError("per-layer stacks (one cache pool per layer) run without KV transfer, KV offload "
+                             "and LoRA")
         if self.stateful:
             from .state_cache import StatePool
 
-            if cfg.kv_transfer_config or cfg.kv_offload_config or cfg.enable_lora:
-                raise ValueError("stateful models run without KV transfer, KV offload and LoRA")
             cfg.cache.enable_prefix_caching = False
             self.state_pool = StatePool(self.model.state_layers(), cfg.sched.max_num_seqs, self.device)
         # KV storage dtype (vLLM --kv-cache-dtype): bf16 or OCP fp8
@@ -182,7 +185,7 @@ class ModelRunner:
         G = self.Hq // self.Hkv
         self.max_window = max((a.window for a in attn if a.window), default=0)
         self.cascade_ok = (cfg.cache.shared_prefix_decode and cfg.cache.enable_prefix_caching and not self.is_mla
-                           and not self.stateful and G <= 16 and 16 % G == 0)
+                           and not self.seq_steps and G <= 16 and 16 % G == 0)
         self.casc_variant = ops.cascade_variant(G, self.D, self.bs, self.kv_dtype != torch.bfloat16) \
             if self.cascade_ok else None
         self.cascade_ok = self.cascade_ok and self.casc_variant is not None
@@ -412,7 +415,7 @@ class ModelRunner:
         return self.num_blocks
 
     def _dummy_prefill(self, T: int, nblocks: int):
-        if self.stateful:  # one sequence of T tokens over the scratch blocks, state slot 0
+        if self.seq_steps:  # one sequence of T tokens over the scratch blocks, state slot 0
             bt = np.zeros((1, self.width), dtype=np.int32)
             nb = math.ceil(T / self.bs)
             bt[0, :nb] = np.arange(nb)
@@ -607,9 +610,9 @@ class ModelRunner:
               "d_len": d_len, "p_ql": p_ql, "p_ctx": p_ctx, "p_bt": p_bt, "rows": rows}
         if self.hybrid:
             pl["swa"] = self._group_tables(so, block_tables.swa)
-        if self.stateful:  # state slot and "continues earlier state" flag per sequence, step order
+        if self.seq_steps:  # state slot and "continues earlier state" flag per sequence, step order
             pl["graph"] = False
-            pl["seq"] = ([block_tables.slots[sr.req.seq_id] for sr in so.all()],
+            pl["seq"] = ([block_tables.slots[sr.req.seq_id] if self.stateful else 0 for sr in so.all()],
                          [int(sr.start > 0) for sr in so.all()])
         if self.lora is not None:
             lo = [sr.req.lora_id for sr in so.decodes]
@@ -963,7 +966,7 @@ class ModelRunner:
 
     @torch.no_grad()
     def capture_graphs(self):
-        if not self.is_gpu or self.cfg.enforce_eager or self.stateful:
+        if not self.is_gpu or self.cfg.enforce_eager or self.seq_steps:
             return
         maxb = min(self.cfg.cuda_graph_max_bs, self.cfg.sched.max_num_seqs)
         buckets = []

@@ -36,6 +36,10 @@ def model_class(cfg: ModelConfig):
         from .mekusun import MekusunForCausalLM
 
         return MekusunForCausalLM
+    if t == "negunex":
+        from .negunex import NegunexForCausalLM
+
+        return NegunexForCausalLM
     raise ValueError(f"unsupported model_type {t!r}")
 
 

@@ -8,6 +8,11 @@ constant is an argument, so another stack can reuse them.
 * ``GeneralDeltaMixer``- generalized delta rule with per-channel decay and removal rate.
 * ``ActMLP`` / ``PlainMoE`` - ungated feed-forwards (xIELU dense; erf-GELU experts with a
   biased fp32 router and softmax over the chosen logits).
+* ``GroupedAttention`` - grouped-query softmax attention with its own key and value sizes, biases,
+  partial rotary (interleaved or half-split pairs, optional frequency scaling), unit-RMS queries and
+  keys, value mixing with an earlier layer and a sigmoid output gate - each one an option.
+* ``GatedMLP`` / ``ScoreMoE`` - gated feed-forwards (act(gate) * up); experts chosen by softmax
+  scores plus a selection-only correction, with identity experts.
 
 Recurrent state lives in the engine's state pool (engine/state_cache.py): a mixer with
 ``state_shapes()`` gets its per-slot tensors through ``bind_state``; the step's
@@ -37,10 +42,20 @@ def _param(shape, device, dtype, std=0.02, fill=None):
     return torch.nn.Parameter(t, requires_grad=False)
 
 
-def rope_table(dims: int, base: float, max_pos: int, device) -> torch.Tensor:
-    """[max_pos, dims] fp32 = [cos(p f_i) | sin(p f_i)], f_i = base^(-2i/dims), angles in fp64."""
+def rope_table(dims: int, base: float, max_pos: int, device, scaling=None) -> torch.Tensor:
+    """[max_pos, dims] fp32 = [cos(p f_i) | sin(p f_i)], f_i = base^(-2i/dims), angles in fp64.
+
+    ``scaling`` = {factor, low, high, original}: frequency scaling by wavelength l = 2 pi / f -
+    f stays where l < original / high, becomes f / factor where l > original / low, and between
+    the two is the blend (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
     half = dims // 2
     f = torch.tensor(base, dtype=torch.float64) ** (-2.0 * torch.arange(half, dtype=torch.float64) / dims)
+    if scaling:
+        fac, lo, hi, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+        wl = 2.0 * math.pi / f
+        s = (orig / wl - lo) / (hi - lo)
+        mid = (1.0 - s) * f / fac + s * f
+        f = torch.where(wl < orig / hi, f, torch.where(wl > orig / lo, f / fac, mid))
     a = torch.arange(max_pos, dtype=torch.float64)[:, None] * f[None]
     return torch.cat([a.cos(), a.sin()], -1).float().to(device)
 
@@ -199,3 +214,117 @@ class PlainMoE(torch.nn.Module):
         logits = F.linear(h.float(), self.router32, self.router_b32)
         ids, w = sm.moe_route(logits, self.k)
         return sm.moe_ffn(h, ids, w, self.w1, self.w2)
+
+
+class GroupedAttention(torch.nn.Module):
+    """Causal softmax attention, ``heads`` query heads over ``kv_heads`` key/value heads, key size
+    ``dim`` and value size ``vdim``. One projection of the layer input gives [q | k | v | gate]; one
+    kernel adds the biases, rotates, normalises, mixes the values and writes the paged cache, whose
+    row per (token, kv head) is [key | value].
+
+    rot          None, or {dims, base, scaling} for rotary positions on the first ``dims`` dimensions
+    interleaved  pairs (2i, 2i+1) instead of (i, i + dims/2)
+    unit_norm    divide rotated q and k by their root mean square over ``dim`` (eps inside the root)
+    v_mix        value mixing: the first such layer of a step publishes its values in
+                 ``shared["v_first"]``; later ones use (1 - vmix) v + vmix v_first, which is what they
+                 cache
+    gate         multiply the concatenated heads by sigmoid(W_g h) before the output projection
+    """
+    is_latent = False
+
+    def __init__(self, d_model, heads, kv_heads, dim, vdim, scale, rot, eps, max_pos, device, dtype, bias=True,
+                 interleaved=True, unit_norm=True, v_mix=False, gate=True):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError(f"{heads} query heads do not divide over {kv_heads} key/value heads")
+        self.Hq, self.Hkv, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.eps, self.interleaved, self.unit_norm = float(scale), eps, interleaved, unit_norm
+        self.v_mix, self.has_gate = bool(v_mix), bool(gate)
+        self.nq, self.nk, self.nv = heads * dim, kv_heads * dim, kv_heads * vdim
+        n = self.nq + self.nk + self.nv + (heads * vdim if gate else 0)
+        self.n_out = -(-n // 8) * 8  # rows of 16-byte multiples for the vector loads downstream
+        self.proj = ColumnLinear(d_model, self.n_out, shard=False, device=device, dtype=dtype)
+        self.bias = _param((self.nq + self.nk + self.nv,), device, dtype, fill=0.0)
+        self.has_bias = bias
+        self.vmix = _param((), device, dtype, fill=0.0)
+        self.o = ColumnLinear(heads * vdim, d_model, shard=False, device=device, dtype=dtype)
+        self.rot_dims = 0
+        if rot:
+            self.rot_dims = int(rot["dims"])
+            if self.rot_dims > dim or self.rot_dims % 2:
+                raise ValueError(f"rotary dims {self.rot_dims} do not fit the head size {dim}")
+            self.register_buffer("cos_sin", rope_table(self.rot_dims, rot["base"], max_pos, device,
+                                                       rot.get("scaling")), persistent=False)
+        else:
+            self.cos_sin = None
+        self.cache = None
+        self.bias32, self.lam = None, 0.0
+        # what the runner's generic bookkeeping reads
+        self.D, self.window, self.sinks = dim + vdim, 0, None
+
+    def finalize(self):
+        self.bias32 = self.bias.data.float()
+        self.lam = float(self.vmix.data.float().item())
+
+    def kv_spec(self):
+        return 1, self.Hkv, self.dim + self.vdim  # (planes, heads, row): [key | value] per kv head
+
+    def bind_cache(self, kv_layer):
+        """kv_layer [blocks, 1, Hkv, bs, dim + vdim] -> [blocks, Hkv, bs, dim + vdim]."""
+        self.cache = kv_layer[:, 0]
+
+    def forward(self, h, meta: AttnMeta, shared=None):
+        T = h.shape[0]
+        p = self.proj(h)
+        q = torch.empty(T, self.Hq, self.dim, dtype=h.dtype, device=h.device)
+        v_first, mode = None, 0
+        if self.v_mix:
+            v_first = shared.get("v_first")
+            mode = 2 if v_first is not None else 1
+            if v_first is None:
+                v_first = shared["v_first"] = torch.empty(T, self.nv, dtype=torch.float32, device=h.device)
+        sm.qkv_rope_cache(p, self.bias32, meta.positions, self.cos_sin, self.Hq, self.Hkv, self.dim, self.vdim,
+                          self.rot_dims, self.interleaved, self.eps if self.unit_norm else None, v_first, mode,
+                          self.lam, meta.slot_mapping, self.cache, q)
+        n0 = self.nq + self.nk + self.nv
+        gate = p[:, n0:n0 + self.Hq * self.vdim] if self.has_gate else None
+        o = sm.grouped_attention(q, self.cache, self.dim, self.vdim, self.scale, meta.seq, gate)
+        return self.o(o)
+
+
+class GatedMLP(torch.nn.Module):
+    """W_down (act(W_gate h) * (W_up h)), gate and up as one projection; act "gelu_tanh" or "silu"."""
+
+    def __init__(self, d_model, ff, act, device, dtype):
+        super().__init__()
+        self.ff, self.act = ff, act
+        self.gate_up = ColumnLinear(d_model, 2 * ff, shard=False, device=device, dtype=dtype)
+        self.down = ColumnLinear(ff, d_model, shard=False, device=device, dtype=dtype)
+
+    def forward(self, h):
+        return self.down(sm.gated_act(self.gate_up(h), self.ff, self.act))
+
+
+class ScoreMoE(torch.nn.Module):
+    """Gated experts chosen by score: router outputs over ``experts + identity`` entries in fp32,
+    scores = softmax over all of them, the ``top`` largest of score + correction chosen, weights = the
+    chosen scores over their sum. The last ``identity`` entries have no weights: they return their
+    input."""
+
+    def __init__(self, d_model, ff, experts, identity, top, act, device, dtype):
+        super().__init__()
+        self.E, self.I, self.k, self.act = experts, identity, top, act
+        self.router = _param((experts + identity, d_model), device, dtype)
+        self.correction = _param((experts + identity,), device, dtype, fill=0.0)
+        self.w1 = _param((experts, 2 * ff, d_model), device, dtype)   # [gate rows | up rows]
+        self.w2 = _param((experts, d_model, ff), device, dtype)
+        self.ff = ff
+        self.router32 = self.correction32 = None
+
+    def finalize(self):
+        self.router32, self.correction32 = self.router.data.float(), self.correction.data.float()
+
+    def forward(self, h):
+        logits = F.linear(h.float(), self.router32)
+        ids, w = sm.moe_route_scores(logits, self.correction32, self.k)
+        return sm.moe_gated_ffn(h, ids, w, self.w1, self.w2, self.act)

@@ -197,10 +197,146 @@ def moe_ffn(h, ids, w, w1, w2):
     C.moe_group(ids, E, slot_row, tile_e, pair_slot)
     a = torch.empty(max_tiles * MOE_TILE, Fh, dtype=h.dtype, device=dev)
     y = torch.empty(max_tiles * MOE_TILE, d, dtype=h.dtype, device=dev)
-    C.moe_gemm(h, k, slot_row, tile_e, w1, a, True, n)   # n = rows of the step: picks the tile width
-    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, False, n)
+    C.moe_gemm(h, k, slot_row, tile_e, w1, a, 1, n)   # n = rows of the step: picks the tile width
+    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, 0, n)
     out = torch.empty_like(h)
-    C.moe_combine(y, pair_slot, w, out)
+    C.moe_combine(y, pair_slot, w, out, None)
+    return out
+
+
+# ---- hyper-connected residual streams
+def hyper_embed(ids, table, X):
+    """X[s] = table[ids] for every stream s (fp32 [S, T, d])."""
+    if not ids.is_cuda:
+        return ref.hyper_embed(ids, table, X)
+    native().hyper_embed(ids, table, X)
+
+
+def hyper_norm(X, w_in, norm_w, eps: float, out_dtype):
+    """Layer norm (weight, no bias; two-pass fp32 variance) of u = sum_s w_in[s] X[s]."""
+    if not X.is_cuda:
+        return ref.hyper_norm(X, w_in, norm_w, eps, out_dtype)
+    out = torch.empty(X.shape[1:], dtype=out_dtype, device=X.device)
+    native().hyper_norm(X, w_in, norm_w, float(eps), out)
+    return out
+
+
+def hyper_update_norm(X, y, mix, w_out, next_in=None, next_w=None, eps: float = 0.0, out_dtype=None):
+    """X[t] <- sum_s mix[s, t] X[s] + w_out[t] y for all streams at once, in place (fp32); with
+    ``next_w`` also returns the layer norm of sum_s next_in[s] X[s], the next sublayer's input (or
+    the model's final norm over the plain sum), from the same pass."""
+    if not X.is_cuda:
+        return ref.hyper_update_norm(X, y, mix, w_out, next_in, next_w, eps, out_dtype)
+    out = torch.empty(X.shape[1:], dtype=out_dtype, device=X.device) if next_w is not None else None
+    native().hyper_update_norm(X, y, mix, w_out, next_in, next_w, float(eps), out)
+    return out
+
+
+# ---- grouped-query attention with its own key and value sizes
+def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps, v_first,
+                   v_mode, lam, slots, cache, q_out):
+    """From a fused projection [q | k | v | ...] of a step's tokens: add ``bias`` (fp32, over q|k|v),
+    rotate the first ``rot_dims`` dimensions of every query and key head by the angles of ``cos_sin``
+    [max_pos, rot_dims] = [cos | sin] (pairs (2i, 2i+1) when ``interleaved``, (i, i + rot_dims/2)
+    otherwise), divide each head by its root mean square (``unit_eps`` not None), mix the values with
+    those of an earlier layer (``v_mode`` 1: store this layer's values in ``v_first`` fp32
+    [T, Hkv * vdim]; 2: v <- (1 - lam) v + lam v_first), write queries to ``q_out`` [T, Hq, dim] and
+    the row [key | value] of every kv head to the paged ``cache`` [blocks, Hkv, bs, dim + vdim] at
+    ``slots`` (-1: no write). All arithmetic fp32."""
+    if not qkv.is_cuda:
+        return ref.qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps,
+                                  v_first, v_mode, lam, slots, cache, q_out)
+    native().qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, bool(interleaved),
+                            unit_eps is not None, float(unit_eps or 0.0), v_first, int(v_mode), float(lam), slots, cache,
+                            q_out)
+
+
+GQA_MFMA = os.environ.get("LLMD_GQA_MFMA", "1") == "1"
+
+
+def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
+    """Causal softmax attention of q [T, Hq, dim] over the paged cache [blocks, Hkv, bs, dim + vdim]
+    (query head h reads kv head h // (Hq / Hkv)); row t sees the first seq.row_len[t] keys of its
+    sequence. ``gate`` [T, Hq * vdim] (a column view of the fused projection): the result is
+    multiplied by sigmoid(gate). Returns [T, Hq * vdim].
+
+    bfloat16 runs on the matrix cores (work item = up to 64 (token, head-of-group) rows of one
+    sequence and kv head); float32 and sizes outside the compiled forms on the fp32 FMA kernel."""
+    T, Hq, _ = q.shape
+    Hkv = cache.shape[1]
+    out = torch.empty(T, Hq * vdim, dtype=q.dtype, device=q.device)
+    if not q.is_cuda:
+        return ref.grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, scale, gate, out)
+    G = Hq // Hkv
+    if GQA_MFMA and q.dtype == torch.bfloat16 and G <= 64:
+        items = seq.attention_items(max(1, 64 // G))
+        nsplit, split, po, pm = 1, 0, None, None
+        if seq.max_q == 1 and seq.max_len > 256:
+            # decode-only step: cut the keys into ranges so that items x kv heads x ranges fill the chip
+            n = items.shape[0] * Hkv
+            nsplit = max(1, min(-(-512 // n), seq.max_len // 128))
+            split = -(-seq.max_len // (nsplit * 32)) * 32
+            nsplit = -(-seq.max_len // split)
+            if nsplit > 1:
+                po = torch.empty(n * nsplit * 64 * vdim, dtype=torch.float32, device=q.device)
+                pm = torch.empty(n * nsplit * 128, dtype=torch.float32, device=q.device)
+        if native().grouped_attention_mfma(q, cache, dim, vdim, seq.tables, items, seq.row_len, float(scale), gate,
+                                           out, nsplit, split, po, pm):
+            return out
+    native().grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, float(scale), gate,
+                               4 if seq.max_q > 1 else 1, out)
+    return out
+
+
+ACT_KINDS = {"gelu_tanh": 0, "silu": 1}
+
+
+def gated_act(gu, Fh: int, kind: str):
+    """act(gu[:, :Fh]) * gu[:, Fh:], act the tanh form of GELU or SiLU, fp32 arithmetic."""
+    if not gu.is_cuda:
+        return ref.gated_act(gu, Fh, kind)
+    out = torch.empty(gu.shape[0], Fh, dtype=gu.dtype, device=gu.device)
+    native().gated_act(gu, int(Fh), ACT_KINDS[kind], out)
+    return out
+
+
+def moe_route_scores(logits, correction, k: int):
+    """Scores = softmax over ALL router outputs (fp32); the k largest of score + correction are
+    chosen (ties: lower index); weights = the chosen scores / (their sum + 1e-20)."""
+    if not logits.is_cuda:
+        return ref.moe_route_scores(logits, correction, k)
+    T = logits.shape[0]
+    ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+    w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    native().moe_route_scores(logits, correction, k, ids, w)
+    return ids, w
+
+
+def moe_gated_ffn(h, ids, w, w1, w2, kind: str = "silu"):
+    """sum_j w[t, j] * W2[e] (act(Wg[e] h_t) * (Wu[e] h_t)), e = ids[t, j]; w1 [E, 2F, d] holds
+    [gate rows | up rows], w2 [E, d, F]. ids >= E name identity experts: their output is h_t itself.
+    Same grouping, tile GEMMs and fp32 combine as ``moe_ffn``; the activation and the product are the
+    first GEMM's epilogue (a workgroup computes matching gate and up columns)."""
+    if not h.is_cuda:
+        return ref.moe_gated_ffn(h, ids, w, w1, w2, kind)
+    C = native()
+    T, d = h.shape
+    k = ids.shape[1]
+    E, F2, _ = w1.shape
+    Fh = F2 // 2
+    n = T * k
+    max_tiles = (n + E * (MOE_TILE - 1)) // MOE_TILE + 1
+    dev = h.device
+    slot_row = torch.empty(max_tiles * MOE_TILE, dtype=torch.int32, device=dev)
+    tile_e = torch.empty(max_tiles, dtype=torch.int32, device=dev)
+    pair_slot = torch.empty(n, dtype=torch.int32, device=dev)       # -1: identity expert
+    C.moe_group(ids, E, slot_row, tile_e, pair_slot)
+    a = torch.empty(max_tiles * MOE_TILE, Fh, dtype=h.dtype, device=dev)
+    y = torch.empty(max_tiles * MOE_TILE, d, dtype=h.dtype, device=dev)
+    C.moe_gemm(h, k, slot_row, tile_e, w1, a, 2 + ACT_KINDS[kind], n)
+    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, 0, n)
+    out = torch.empty_like(h)
+    C.moe_combine(y, pair_slot, w, out, h)
     return out
 
 

@@ -149,3 +149,110 @@ def moe_ffn(h, ids, w, w1, w2):
 
 def softcap_(logits, cap):
     return logits.copy_(cap * torch.tanh(logits / cap))
+
+
+# ---- hyper-connected streams, grouped attention with separate key / value sizes, gated feed-forwards
+def _ln(u, w, eps):
+    u = u.float()
+    dev = u - u.mean(-1, keepdim=True)
+    return dev * torch.rsqrt(dev.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+
+def hyper_embed(ids, table, X):
+    X.copy_(table[ids].float().unsqueeze(0).expand_as(X))
+
+
+def hyper_norm(X, w_in, norm_w, eps, out_dtype):
+    return _ln((X * w_in.view(-1, 1, 1)).sum(0), norm_w, eps).to(out_dtype)
+
+
+def hyper_update_norm(X, y, mix, w_out, next_in, next_w, eps, out_dtype):
+    new = torch.einsum("st,snd->tnd", mix, X) + w_out.view(-1, 1, 1) * y.float().unsqueeze(0)
+    X.copy_(new)
+    return None if next_w is None else hyper_norm(X, next_in, next_w, eps, out_dtype)
+
+
+def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps, v_first,
+                   v_mode, lam, slots, cache, q_out):
+    T = qkv.shape[0]
+    nq, nk, nv = Hq * dim, Hkv * dim, Hkv * vdim
+    x = qkv[:, :nq + nk + nv].float() + bias.float()
+    q, k, v = x[:, :nq].view(T, Hq, dim), x[:, nq:nq + nk].view(T, Hkv, dim), x[:, nq + nk:].view(T, Hkv, vdim)
+    if rot_dims:
+        half = rot_dims // 2
+        cs = cos_sin[positions]
+        c, s = cs[:, None, :half], cs[:, None, half:]
+
+        def rot(t):
+            if interleaved:
+                a, b = t[..., 0:rot_dims:2], t[..., 1:rot_dims:2]
+                r = torch.stack([a * c - b * s, b * c + a * s], -1).flatten(-2)
+            else:
+                a, b = t[..., :half], t[..., half:rot_dims]
+                r = torch.cat([a * c - b * s, b * c + a * s], -1)
+            return torch.cat([r, t[..., rot_dims:]], -1)
+
+        q, k = rot(q), rot(k)
+    if unit_eps is not None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + unit_eps)
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + unit_eps)
+    if v_mode == 1:
+        v_first.copy_(v.reshape(T, nv))
+    elif v_mode == 2:
+        v = (1.0 - lam) * v + lam * v_first.view(T, Hkv, vdim)
+    q_out.copy_(q.to(q_out.dtype))
+    row = torch.cat([k, v], -1).to(cache.dtype)              # [T, Hkv, dim + vdim]
+    nb, _, bs, _ = cache.shape
+    ok = slots >= 0
+    sl = slots[ok]
+    cache[sl // bs, :, sl % bs] = row[ok]
+
+
+def grouped_attention(q, cache, dim, vdim, tables, row_seq, row_len, scale, gate, out):
+    T, Hq, _ = q.shape
+    nb, Hkv, bs, _ = cache.shape
+    G = Hq // Hkv
+    for t in range(T):
+        n = int(row_len[t])
+        bt = tables[int(row_seq[t])].long()
+        ar = torch.arange(n)
+        rows = cache[bt[ar // bs], :, ar % bs].float()        # [n, Hkv, dim + vdim]
+        K, V = rows[..., :dim], rows[..., dim:]
+        qt = q[t].float().view(Hkv, G, dim)
+        s = torch.einsum("hgd,nhd->hgn", qt, K) * scale
+        o = torch.einsum("hgn,nhv->hgv", torch.softmax(s, -1), V).reshape(Hq * vdim)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t].float())
+        out[t] = o.to(out.dtype)
+    return out
+
+
+def _act(z, kind):
+    return F.gelu(z, approximate="tanh") if kind == "gelu_tanh" else F.silu(z)
+
+
+def gated_act(gu, Fh, kind):
+    return (_act(gu[:, :Fh].float(), kind) * gu[:, Fh:].float()).to(gu.dtype)
+
+
+def moe_route_scores(logits, correction, k):
+    s = torch.softmax(logits.float(), -1)
+    ids = (s + correction.float()).topk(k, -1).indices
+    w = torch.gather(s, 1, ids)
+    return ids.int(), w / (w.sum(-1, keepdim=True) + 1e-20)
+
+
+def moe_gated_ffn(h, ids, w, w1, w2, kind):
+    """w1 [E, 2F, d] = [gate | up] rows, w2 [E, d, F]; ids >= E are identity experts."""
+    E, F2, _ = w1.shape
+    out = torch.zeros(h.shape, dtype=torch.float32)
+    hf = h.float()
+    for e in ids.unique().tolist():
+        t, j = (ids == e).nonzero(as_tuple=True)
+        if e >= E:
+            out.index_add_(0, t, hf[t] * w[t, j, None])
+            continue
+        gu = (hf[t] @ w1[e].float().T)
+        a = (_act(gu[:, :F2 // 2], kind) * gu[:, F2 // 2:]).to(h.dtype).float()
+        out.index_add_(0, t, (a @ w2[e].float().T).to(h.dtype).float() * w[t, j, None])
+    return out.to(h.dtype)
