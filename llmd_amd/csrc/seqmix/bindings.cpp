@@ -28,11 +28,23 @@ int sm_selective_scan(const void*, const void*, const void*, const float*, const
                       hipStream_t);
 int sm_gdelta_scan(const void*, int64_t, const void*, const void*, const void*, const void*, float, int, int, float*,
                    const int*, const int*, const int*, void*, int, int, hipStream_t);
+void sm_hyper_embed(const int64_t*, const void*, int64_t, float*, int, int, int, int, hipStream_t);
+void sm_hyper_norm(const float*, const float*, const void*, float, void*, int, int, int, int, hipStream_t);
+void sm_hyper_update_norm(float*, const void*, int64_t, const float*, const float*, const float*, const void*, float,
+                          void*, int, int, int, int, hipStream_t);
+void sm_gated_act(const void*, int64_t, int, int, void*, int, int, hipStream_t);
+void sm_qkv_rope_cache(const void*, int64_t, const float*, const int64_t*, const float*, int, int, int, int, int, int,
+                       int, float, float*, int, float, const int64_t*, void*, int, void*, int, int, hipStream_t);
+int sm_grouped_attention(const void*, const void*, const int*, int, int, const int*, const int*, float, int, int, int,
+                         int, int, int, const void*, int64_t, void*, int, hipStream_t);
+int sm_grouped_attention_mfma(const void*, const void*, const int*, int, int, const int*, int, const int*, float, int,
+                              int, int, int, const void*, int64_t, void*, int, int, float*, float*, hipStream_t);
+void sm_moe_route_scores(const float*, const float*, int, int, int*, float*, int, hipStream_t);
 void sm_moe_route(const float*, int, int, int*, float*, int, hipStream_t);
 void sm_moe_group(const int*, int, int, int*, int*, int*, int, hipStream_t);
 void sm_moe_gemm(const void*, int64_t, int, const int*, const int*, const void*, int, int, void*, int, int, int, int,
                  hipStream_t);
-void sm_moe_combine(const void*, const int*, const float*, int, int, void*, int, int, hipStream_t);
+void sm_moe_combine(const void*, const int*, const float*, int, int, void*, const void*, int, int, hipStream_t);
 }
 
 namespace {
@@ -286,6 +298,183 @@ void gdelta_scan(Tensor proj, Tensor wl, Tensor w0, Tensor a_b, Tensor norm_w, d
   TORCH_CHECK(rc == 0, "gdelta_scan: head size above 256");
 }
 
+void hyper_embed(Tensor ids, Tensor table, Tensor X) {
+  const c10::hip::OptionalHIPGuard g(dev_of(ids));
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == torch::kInt64 && ids.is_contiguous(), "ids: int64");
+  TORCH_CHECK(table.is_cuda() && act_ok(table) && table.dim() == 2 && table.is_contiguous(), "table");
+  CHECK_F32(X);
+  const int T = ids.numel(), d = table.size(1);
+  TORCH_CHECK(X.dim() == 3 && X.size(0) >= 1 && X.size(0) <= 8 && X.size(1) == T && X.size(2) == d, "X [S <= 8, T, d]");
+  sm_hyper_embed(ids.data_ptr<int64_t>(), table.data_ptr(), table.size(0), X.data_ptr<float>(), X.size(0), T, d,
+                 is_f32(table), cur());
+}
+
+void check_streams(const Tensor& X) {
+  CHECK_F32(X);
+  TORCH_CHECK(X.dim() == 3 && X.size(0) >= 1 && X.size(0) <= 8 && X.size(2) <= 16384, "X [S <= 8, T, d <= 16384]");
+}
+
+void hyper_norm(Tensor X, Tensor w_in, Tensor norm_w, double eps, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(X));
+  check_streams(X);
+  CHECK_F32(w_in);
+  const int S = X.size(0), T = X.size(1), d = X.size(2);
+  TORCH_CHECK(w_in.numel() == S && norm_w.is_cuda() && act_ok(norm_w) && norm_w.is_contiguous() && norm_w.numel() == d,
+              "weights");
+  CHECK_ACT(out, norm_w);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == d, "out [T, d]");
+  sm_hyper_norm(X.data_ptr<float>(), w_in.data_ptr<float>(), norm_w.data_ptr(), (float)eps, out.data_ptr(), S, T, d,
+                is_f32(norm_w), cur());
+}
+
+void hyper_update_norm(Tensor X, Tensor y, Tensor mix, Tensor w_out, std::optional<Tensor> next_in,
+                       std::optional<Tensor> next_w, double eps, std::optional<Tensor> out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(X));
+  check_streams(X);
+  CHECK_F32(mix);
+  CHECK_F32(w_out);
+  const int S = X.size(0), T = X.size(1), d = X.size(2);
+  TORCH_CHECK(y.is_cuda() && act_ok(y) && y.dim() == 2 && y.size(0) == T && y.size(1) == d && y.stride(1) == 1, "y [T, d]");
+  TORCH_CHECK(mix.numel() == (int64_t)S * S && w_out.numel() == S, "mix [S, S], out [S]");
+  const float* nin = nullptr;
+  const void* nw = nullptr;
+  void* o = nullptr;
+  if (next_w) {
+    TORCH_CHECK(next_in && out, "next_in and out come with next_w");
+    CHECK_F32(*next_in);
+    CHECK_ACT(*next_w, y);
+    CHECK_ACT(*out, y);
+    TORCH_CHECK(next_in->numel() == S && next_w->is_contiguous() && next_w->numel() == d && out->is_contiguous() &&
+                    out->dim() == 2 && out->size(0) == T && out->size(1) == d, "next norm shapes");
+    nin = next_in->data_ptr<float>();
+    nw = next_w->data_ptr();
+    o = out->data_ptr();
+  }
+  sm_hyper_update_norm(X.data_ptr<float>(), y.data_ptr(), y.stride(0), mix.data_ptr<float>(), w_out.data_ptr<float>(),
+                       nin, nw, (float)eps, o, S, T, d, is_f32(y), cur());
+}
+
+void gated_act(Tensor gu, int64_t F, int64_t kind, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(gu));
+  TORCH_CHECK(gu.is_cuda() && act_ok(gu) && gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) >= 2 * F && F >= 1, "gu");
+  CHECK_ACT(out, gu);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == gu.size(0) && out.size(1) == F &&
+                  (kind == 0 || kind == 1), "out [T, F]");
+  sm_gated_act(gu.data_ptr(), gu.stride(0), F, kind, out.data_ptr(), gu.size(0), is_f32(gu), cur());
+}
+
+void qkv_rope_cache(Tensor qkv, std::optional<Tensor> bias, Tensor positions, std::optional<Tensor> cos_sin, int64_t Hq,
+                    int64_t Hkv, int64_t dim, int64_t vdim, int64_t rot_dims, bool interleaved, bool unit, double eps,
+                    std::optional<Tensor> v_first, int64_t v_mode, double lam, Tensor slots, Tensor cache,
+                    Tensor q_out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(qkv));
+  TORCH_CHECK(qkv.is_cuda() && act_ok(qkv) && qkv.dim() == 2 && qkv.stride(1) == 1, "qkv");
+  const int64_t T = qkv.size(0), n = (Hq + Hkv) * dim + Hkv * vdim;
+  TORCH_CHECK(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0 && dim >= 1 && dim <= 512 && vdim >= 1 && qkv.size(1) >= n, "sizes");
+  TORCH_CHECK(rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0, "rotary dims");
+  TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == torch::kInt64 && positions.is_contiguous() &&
+                  positions.numel() == T && slots.is_cuda() && slots.scalar_type() == torch::kInt64 &&
+                  slots.is_contiguous() && slots.numel() == T, "positions / slots: int64 [T]");
+  if (bias) {
+    CHECK_F32(*bias);
+    TORCH_CHECK(bias->numel() == n, "bias over q | k | v");
+  }
+  if (rot_dims) {
+    TORCH_CHECK(cos_sin.has_value(), "cos_sin");
+    CHECK_F32(*cos_sin);
+    TORCH_CHECK(cos_sin->dim() == 2 && cos_sin->size(1) == rot_dims, "cos_sin [max_pos, rot_dims]");
+  }
+  TORCH_CHECK(v_mode >= 0 && v_mode <= 2, "v_mode");
+  if (v_mode) {
+    TORCH_CHECK(v_first.has_value(), "v_first");
+    CHECK_F32(*v_first);
+    TORCH_CHECK(v_first->numel() == T * Hkv * vdim, "v_first [T, Hkv * vdim]");
+  }
+  CHECK_ACT(cache, qkv);
+  CHECK_ACT(q_out, qkv);
+  TORCH_CHECK(cache.dim() == 4 && cache.is_contiguous() && cache.size(1) == Hkv && cache.size(3) == dim + vdim,
+              "cache [blocks, Hkv, bs, dim + vdim]");
+  TORCH_CHECK(q_out.is_contiguous() && q_out.numel() == T * Hq * dim, "q_out [T, Hq, dim]");
+  sm_qkv_rope_cache(qkv.data_ptr(), qkv.stride(0), bias ? bias->data_ptr<float>() : nullptr,
+                    positions.data_ptr<int64_t>(), rot_dims ? cos_sin->data_ptr<float>() : nullptr, Hq, Hkv, dim, vdim,
+                    rot_dims, interleaved ? 1 : 0, unit ? 1 : 0, (float)eps, v_mode ? v_first->data_ptr<float>() : nullptr,
+                    v_mode, (float)lam, slots.data_ptr<int64_t>(), cache.data_ptr(), cache.size(2), q_out.data_ptr(), T,
+                    is_f32(qkv), cur());
+}
+
+void check_gqa(const Tensor& q, const Tensor& cache, int64_t dim, int64_t vdim, const Tensor& tables,
+               const Tensor& row_len, const std::optional<Tensor>& gate, const Tensor& out) {
+  TORCH_CHECK(q.is_cuda() && act_ok(q) && q.dim() == 3 && q.is_contiguous() && q.size(2) == dim, "q [T, Hq, dim]");
+  CHECK_ACT(cache, q);
+  CHECK_ACT(out, q);
+  TORCH_CHECK(cache.dim() == 4 && cache.is_contiguous() && cache.size(3) == dim + vdim && q.size(1) % cache.size(1) == 0,
+              "cache [blocks, Hkv, bs, dim + vdim]");
+  CHECK_I32(tables);
+  CHECK_I32(row_len);
+  TORCH_CHECK(tables.dim() == 2 && row_len.numel() == q.size(0), "tables [n, W], row_len [T]");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == q.size(0) * q.size(1) * vdim, "out [T, Hq * vdim]");
+  if (gate) {
+    CHECK_ACT(*gate, q);
+    TORCH_CHECK(gate->dim() == 2 && gate->size(0) == q.size(0) && gate->size(1) == q.size(1) * vdim &&
+                    gate->stride(1) == 1, "gate [T, Hq * vdim]");
+  }
+}
+
+void grouped_attention(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor tables, Tensor row_seq, Tensor row_len,
+                       double scale, std::optional<Tensor> gate, int64_t rows_per_group, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(q));
+  check_gqa(q, cache, dim, vdim, tables, row_len, gate, out);
+  CHECK_I32(row_seq);
+  TORCH_CHECK(row_seq.numel() == q.size(0) && (rows_per_group == 1 || rows_per_group == 4), "row_seq [T]");
+  const int rc = sm_grouped_attention(q.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
+                                      cache.size(2), row_seq.data_ptr<int>(), row_len.data_ptr<int>(), (float)scale,
+                                      q.size(1), cache.size(1), dim, vdim, q.size(0), rows_per_group,
+                                      gate ? gate->data_ptr() : nullptr, gate ? gate->stride(0) : 0, out.data_ptr(),
+                                      is_f32(q), cur());
+  TORCH_CHECK(rc == 0, "grouped_attention: head sizes too large for the kernel (vdim <= 1024, one key tile in LDS)");
+}
+
+bool grouped_attention_mfma(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor tables, Tensor items,
+                            Tensor row_len, double scale, std::optional<Tensor> gate, Tensor out, int64_t nsplit,
+                            int64_t split_keys, std::optional<Tensor> part_o, std::optional<Tensor> part_ml) {
+  const c10::hip::OptionalHIPGuard g(dev_of(q));
+  check_gqa(q, cache, dim, vdim, tables, row_len, gate, out);
+  TORCH_CHECK(q.scalar_type() == torch::kBFloat16, "bf16 only");
+  CHECK_I32(items);
+  TORCH_CHECK(items.dim() == 2 && items.size(1) == 3, "items [n, 3]");
+  const int64_t n = items.size(0), Hkv = cache.size(1);
+  float *po = nullptr, *pm = nullptr;
+  TORCH_CHECK(nsplit >= 1, "nsplit");
+  if (nsplit > 1) {
+    TORCH_CHECK(part_o && part_ml && split_keys > 0 && split_keys % 32 == 0, "split workspace");
+    CHECK_F32(*part_o);
+    CHECK_F32(*part_ml);
+    TORCH_CHECK(part_o->numel() >= n * Hkv * nsplit * 64 * vdim && part_ml->numel() >= n * Hkv * nsplit * 128,
+                "split workspace too small");
+    po = part_o->data_ptr<float>();
+    pm = part_ml->data_ptr<float>();
+  }
+  const int rc = sm_grouped_attention_mfma(q.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
+                                           cache.size(2), items.data_ptr<int>(), n, row_len.data_ptr<int>(),
+                                           (float)scale, q.size(1), Hkv, dim, vdim, gate ? gate->data_ptr() : nullptr,
+                                           gate ? gate->stride(0) : 0, out.data_ptr(), nsplit, split_keys, po, pm,
+                                           cur());
+  return rc == 0;
+}
+
+void moe_route_scores(Tensor logits, Tensor correction, int64_t k, Tensor ids, Tensor w) {
+  const c10::hip::OptionalHIPGuard g(dev_of(logits));
+  CHECK_F32(logits);
+  CHECK_F32(correction);
+  CHECK_I32(ids);
+  CHECK_F32(w);
+  const int T = logits.size(0), E = logits.size(1);
+  TORCH_CHECK(logits.dim() == 2 && k >= 1 && k <= E && correction.numel() == E && ids.numel() == (int64_t)T * k &&
+                  w.numel() == (int64_t)T * k, "router shapes");
+  sm_moe_route_scores(logits.data_ptr<float>(), correction.data_ptr<float>(), E, k, ids.data_ptr<int>(),
+                      w.data_ptr<float>(), T, cur());
+}
+
 void moe_route(Tensor logits, int64_t k, Tensor ids, Tensor w) {
   const c10::hip::OptionalHIPGuard g(dev_of(logits));
   CHECK_F32(logits);
@@ -310,7 +499,7 @@ void moe_group(Tensor ids, int64_t E, Tensor slot_row, Tensor tile_e, Tensor pai
                mt, cur());
 }
 
-void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, Tensor C, bool gelu, int64_t rows) {
+void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, Tensor C, int64_t act, int64_t rows) {
   const c10::hip::OptionalHIPGuard g(dev_of(A));
   TORCH_CHECK(A.is_cuda() && act_ok(A) && A.dim() == 2 && A.stride(1) == 1, "A");
   CHECK_ACT(W, A);
@@ -319,14 +508,16 @@ void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, 
   CHECK_I32(tile_e);
   TORCH_CHECK(W.dim() == 3 && W.is_contiguous() && W.size(2) == A.size(1), "W [E, N, K]");
   const int64_t mt = tile_e.numel();
+  TORCH_CHECK(act >= 0 && act <= 3 && (act < 2 || W.size(1) % 2 == 0), "epilogue");
+  const int64_t N = act >= 2 ? W.size(1) / 2 : W.size(1);  // gated: W holds [gate rows | up rows]
   TORCH_CHECK(slot_row.numel() == mt * 64 && C.is_contiguous() && C.dim() == 2 && C.size(0) == mt * 64 &&
-                  C.size(1) == W.size(1), "C [tiles * 64, N]");
+                  C.size(1) == N, "C [tiles * 64, N]");
   TORCH_CHECK(kdiv > 0 || A.size(0) == mt * 64, "A rows are the tile slots");
   sm_moe_gemm(A.data_ptr(), A.stride(0), kdiv, slot_row.data_ptr<int>(), tile_e.data_ptr<int>(), W.data_ptr(),
-              W.size(1), W.size(2), C.data_ptr(), mt, rows, gelu ? 1 : 0, is_f32(A), cur());
+              N, W.size(2), C.data_ptr(), mt, rows, (int)act, is_f32(A), cur());
 }
 
-void moe_combine(Tensor y, Tensor pair_slot, Tensor w, Tensor out) {
+void moe_combine(Tensor y, Tensor pair_slot, Tensor w, Tensor out, std::optional<Tensor> h) {
   const c10::hip::OptionalHIPGuard g(dev_of(y));
   TORCH_CHECK(y.is_cuda() && act_ok(y) && y.dim() == 2 && y.is_contiguous(), "y");
   CHECK_I32(pair_slot);
@@ -335,8 +526,13 @@ void moe_combine(Tensor y, Tensor pair_slot, Tensor w, Tensor out) {
   const int T = out.size(0), d = out.size(1);
   TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && y.size(1) == d && w.dim() == 2 && w.size(0) == T &&
                   pair_slot.numel() == w.numel(), "combine shapes");
-  sm_moe_combine(y.data_ptr(), pair_slot.data_ptr<int>(), w.data_ptr<float>(), w.size(1), d, out.data_ptr(), T,
-                 is_f32(y), cur());
+  // h: the tokens' inputs, read for pairs marked -1 (identity experts); without it no pair may be -1
+  if (h) {
+    CHECK_ACT(*h, y);
+    TORCH_CHECK(h->dim() == 2 && h->is_contiguous() && h->size(0) == T && h->size(1) == d, "h [T, d]");
+  }
+  sm_moe_combine(y.data_ptr(), pair_slot.data_ptr<int>(), w.data_ptr<float>(), w.size(1), d, out.data_ptr(),
+                 h ? h->data_ptr() : y.data_ptr(), T, is_f32(y), cur());
 }
 
 }  // namespace
@@ -354,6 +550,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("causal_conv_silu", &causal_conv_silu);
   m.def("selective_scan", &selective_scan);
   m.def("gdelta_scan", &gdelta_scan);
+  m.def("hyper_embed", &hyper_embed);
+  m.def("hyper_norm", &hyper_norm);
+  m.def("hyper_update_norm", &hyper_update_norm);
+  m.def("gated_act", &gated_act);
+  m.def("qkv_rope_cache", &qkv_rope_cache);
+  m.def("grouped_attention", &grouped_attention);
+  m.def("grouped_attention_mfma", &grouped_attention_mfma);
+  m.def("moe_route_scores", &moe_route_scores);
   m.def("moe_route", &moe_route);
   m.def("moe_group", &moe_group);
   m.def("moe_gemm", &moe_gemm);

@@ -1,0 +1,545 @@
+// Grouped-query softmax attention with separate key and value sizes over a paged cache whose
+// row per (token, kv head) is [key (dim) | value (vdim)]: cache [blocks, Hkv, bs, dim + vdim].
+//
+// qkv_rope_cache: one workgroup per token over the fused projection [q | k | v | ...]: bias add,
+//   rotary on the first rot_dims dimensions of every q and k head (pairs (2i, 2i+1) or
+//   (i, i + rot_dims/2); angles from an fp32 [cos | sin] table), division of each head by its
+//   root mean square, value mixing with an earlier layer's values, query and cache writes. A wave
+//   owns a head (its elements in registers); everything is fp32 until the store.
+// grouped_attention (fp32 FMA form): workgroup = QT consecutive token rows x up to 4 query heads
+//   of ONE kv head (a wave per head). Keys and values stream through LDS in fp32 tiles; a lane
+//   scores one key, the wave keeps an online softmax per (row, head), lanes then own value columns.
+// grouped_attention_mfma (bf16): a workgroup takes one work item - up to 64 (token, head of the
+//   group) rows of one sequence and kv head, 16 rows per wave. Key tiles of 32 in LDS (keys
+//   row-major, values transposed), S^T = K Q^T and O += P V on v_mfma_f32_16x16x32_bf16; fp32
+//   online softmax; P enters the second product as a bf16 pair (hi + lo). Decode-only steps cut
+//   the keys into ranges over blockIdx.z and a merge kernel joins them.
+// Both forms multiply the result by sigmoid(gate) when a gate is given. A row's result depends
+// only on its own keys and the fixed tile sizes.
+#include "seqmix_common.h"
+
+using namespace sm;
+
+namespace {
+
+constexpr int NT = 256;
+constexpr int MAXE = 8;  // head elements per lane: dim <= 512
+
+template <typename T>
+__global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
+    const T* __restrict__ qkv, int64_t stride, const float* __restrict__ bias, const int64_t* __restrict__ positions,
+    const float* __restrict__ cos_sin, int Hq, int Hkv, int dim, int vdim, int rot_dims, int interleaved, int unit,
+    float eps, float* __restrict__ v_first, int v_mode, float lam, const int64_t* __restrict__ slots,
+    T* __restrict__ cache, int bs, T* __restrict__ q_out) {
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int half = rot_dims >> 1;
+  const float* cs = rot_dims ? cos_sin + positions[t] * rot_dims : nullptr;  // [cos(half) | sin(half)]
+  const T* row = qkv + t * stride;
+  const int64_t slot = slots[t];
+  const int Dr = dim + vdim;
+  const int64_t blk = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
+  for (int hd = wave; hd < Hq + Hkv; hd += NT / 64) {
+    const bool is_q = hd < Hq;
+    const int col0 = is_q ? hd * dim : Hq * dim + (hd - Hq) * dim;
+    float r[MAXE];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXE; ++i) {
+      const int e = lane + 64 * i;
+      float v = 0.f;
+      if (e < dim) {
+        const float x = ld(row + col0 + e) + (bias ? bias[col0 + e] : 0.f);
+        v = x;
+        if (e < rot_dims) {
+          int p, f;
+          bool first;
+          if (interleaved) {
+            p = e ^ 1;
+            f = e >> 1;
+            first = (e & 1) == 0;
+          } else {
+            first = e < half;
+            p = first ? e + half : e - half;
+            f = first ? e : e - half;
+          }
+          const float xp = ld(row + col0 + p) + (bias ? bias[col0 + p] : 0.f);
+          const float c = cs[f], s = cs[half + f];
+          v = first ? x * c - xp * s : x * c + xp * s;
+        }
+      }
+      r[i] = v;
+      ss += v * v;
+    }
+    float inv = 1.f;
+    if (unit) inv = 1.f / sqrtf(wave_sum(ss) / (float)dim + eps);
+    T* dst = nullptr;
+    if (is_q) dst = q_out + (t * Hq + hd) * dim;
+    else if (slot >= 0) dst = cache + ((blk * Hkv + (hd - Hq)) * bs + off) * Dr;
+    if (dst == nullptr) continue;
+#pragma unroll
+    for (int i = 0; i < MAXE; ++i) {
+      const int e = lane + 64 * i;
+      if (e < dim) st(dst + e, r[i] * inv);
+    }
+  }
+  const int nv = Hkv * vdim, vcol0 = (Hq + Hkv) * dim;
+  for (int e = threadIdx.x; e < nv; e += NT) {
+    float v = ld(row + vcol0 + e) + (bias ? bias[vcol0 + e] : 0.f);
+    if (v_mode == 1) v_first[t * nv + e] = v;
+    else if (v_mode == 2) v = (1.f - lam) * v + lam * v_first[t * nv + e];
+    if (slot >= 0) {
+      const int g = e / vdim, c = e - g * vdim;
+      st(cache + ((blk * Hkv + g) * bs + off) * Dr + dim + c, v);
+    }
+  }
+}
+
+// VC = ceil(vdim / 64) output columns per lane; QT token rows per workgroup.
+template <typename T, int VC, int QT>
+__global__ __launch_bounds__(NT) void grouped_attention_kernel(
+    const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
+    const int* __restrict__ row_seq, const int* __restrict__ row_len, float scale, int Hq, int Hkv, int dim, int vdim,
+    int KT, int T_rows, const T* __restrict__ gate, int64_t gate_stride, T* __restrict__ out) {
+  extern __shared__ float lds[];
+  const int Dr = dim + vdim;
+  const int KS = Dr + 1;                 // tile row stride (odd: lanes hit distinct banks)
+  float* sK = lds;                       // [KT][KS]  key | value
+  float* sQ = lds + KT * KS;             // [QT][4][dim], pre-scaled
+  const int G = Hq / Hkv, subs = (G + 3) / 4;
+  const int g = blockIdx.y / subs, sub = blockIdx.y - g * subs;
+  const int t0 = blockIdx.x * QT;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int hg = sub * 4 + wave;         // head within the group
+  const bool head_ok = hg < G;
+  const int h = g * G + hg;
+
+  for (int e = threadIdx.x; e < QT * 4 * dim; e += NT) {
+    const int r = e / (4 * dim), rem = e - r * 4 * dim;
+    const int w = rem / dim, d = rem - w * dim;
+    const int t = t0 + r, hh = sub * 4 + w;
+    sQ[e] = (t < T_rows && hh < G) ? ld(q + ((int64_t)t * Hq + g * G + hh) * dim + d) * scale : 0.f;
+  }
+
+  int seq_r[QT], len_r[QT];
+  bool done[QT];
+#pragma unroll
+  for (int r = 0; r < QT; ++r) {
+    const int t = t0 + r;
+    done[r] = t >= T_rows;
+    seq_r[r] = done[r] ? -1 : row_seq[t];
+    len_r[r] = done[r] ? 0 : row_len[t];
+  }
+
+  for (int pass = 0; pass < QT; ++pass) {
+    int seq = -1;
+#pragma unroll
+    for (int r = 0; r < QT; ++r)
+      if (seq < 0 && !done[r]) seq = seq_r[r];
+    if (seq < 0) break;
+    bool act[QT];
+    int maxlen = 0;
+#pragma unroll
+    for (int r = 0; r < QT; ++r) {
+      act[r] = !done[r] && seq_r[r] == seq;
+      if (act[r]) maxlen = max(maxlen, len_r[r]);
+    }
+    float m[QT], l[QT], acc[QT][VC];
+#pragma unroll
+    for (int r = 0; r < QT; ++r) {
+      m[r] = -INFINITY;
+      l[r] = 0.f;
+#pragma unroll
+      for (int c = 0; c < VC; ++c) acc[r][c] = 0.f;
+    }
+    const int* bt = tables + (int64_t)seq * W;
+    for (int k0 = 0; k0 < maxlen; k0 += KT) {
+      __syncthreads();  // previous tile fully used (and sQ written, first time)
+      for (int e = threadIdx.x; e < KT * Dr; e += NT) {
+        const int j = e / Dr, d = e - j * Dr;
+        const int key = k0 + j;
+        float v = 0.f;
+        if (key < maxlen) {
+          const int64_t rowi = ((int64_t)bt[key / bs] * Hkv + g) * bs + (key % bs);
+          v = ld(cache + rowi * Dr + d);
+        }
+        sK[j * KS + d] = v;
+      }
+      __syncthreads();
+      if (!head_ok) continue;
+#pragma unroll
+      for (int r = 0; r < QT; ++r) {
+        if (!act[r] || k0 >= len_r[r]) continue;
+        const bool valid = lane < KT && k0 + lane < len_r[r];
+        float s = -INFINITY;
+        if (valid) {
+          const float* qv = sQ + (r * 4 + wave) * dim;
+          const float* kr = sK + lane * KS;
+          float a = 0.f;
+          for (int d = 0; d < dim; ++d) a += qv[d] * kr[d];
+          s = a;
+        }
+        const float mn = fmaxf(m[r], wave_max(s));
+        const float corr = expf(m[r] - mn);  // exp(-inf) = 0 on the first tile
+        const float p = valid ? expf(s - mn) : 0.f;
+        l[r] = l[r] * corr + wave_sum(p);
+        m[r] = mn;
+#pragma unroll
+        for (int c = 0; c < VC; ++c) acc[r][c] *= corr;
+        const int nk = min(KT, len_r[r] - k0);
+        for (int j = 0; j < nk; ++j) {
+          const float pj = __shfl(p, j, 64);
+          const float* vr = sK + j * KS + dim;
+#pragma unroll
+          for (int c = 0; c < VC; ++c) {
+            const int col = lane + 64 * c;
+            if (col < vdim) acc[r][c] += pj * vr[col];
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < QT; ++r) {
+      if (!act[r]) continue;
+      done[r] = true;
+      if (!head_ok) continue;
+      const float inv = 1.f / l[r];
+#pragma unroll
+      for (int c = 0; c < VC; ++c) {
+        const int col = lane + 64 * c;
+        if (col >= vdim) continue;
+        float o = acc[r][c] * inv;
+        if (gate) o *= 1.f / (1.f + expf(-ld(gate + (int64_t)(t0 + r) * gate_stride + h * vdim + col)));
+        st(out + ((int64_t)(t0 + r) * Hq + h) * vdim + col, o);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int MKT = 32;  // keys per tile
+
+// DkP = 32 NKS >= dim and VP = 16 NCB >= vdim are the padded sizes (zeros in LDS and in the
+// query fragments). items [n, 3] = (sequence, first token row, tokens), tokens * G <= 64.
+template <int NKS, int NCB>
+__global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
+    const int* __restrict__ items, const int* __restrict__ row_len, float scale, int Hq, int Hkv, int dim, int vdim,
+    const bf16_t* __restrict__ gate, int64_t gate_stride, bf16_t* __restrict__ out, int split_keys,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
+  constexpr int DkP = 32 * NKS, VP = 16 * NCB;
+  constexpr int KS = DkP + 8, VS = MKT + 8, PS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
+  __shared__ __attribute__((aligned(16))) bf16_t sK[MKT * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t sVt[VP * VS];
+  __shared__ __attribute__((aligned(16))) bf16_t sP[2 * 4 * 16 * PS];
+  bf16_t* const sPh = sP;
+  bf16_t* const sPl = sP + 4 * 16 * PS;
+  const int seq = items[blockIdx.x * 3], tok0 = items[blockIdx.x * 3 + 1], ntok = items[blockIdx.x * 3 + 2];
+  const int g = blockIdx.y, G = Hq / Hkv, Dr = dim + vdim;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, kq = lane >> 4;
+  // this lane's query row (as the B operand's column): item row 16 wave + r16
+  const int myrow = wave * 16 + r16;
+  const bool row_ok = myrow < ntok * G;
+  const int mytok = tok0 + (row_ok ? myrow / G : 0), myhead = g * G + (row_ok ? myrow % G : 0);
+  const int mylen = row_ok ? row_len[mytok] : 0;
+  const int maxlen = row_len[tok0 + ntok - 1];  // the run's last token sees the most keys
+
+  // padding columns of the key tile and padding rows of the value tile stay zero for the whole kernel
+  for (int e = threadIdx.x; e < MKT * KS; e += NT) sK[e] = 0;
+  for (int e = threadIdx.x; e < VP * VS; e += NT) sVt[e] = 0;
+
+  bf16x8_t qf[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int d = ks * 32 + kq * 8 + i;
+      const bf16_t w = (row_ok && d < dim) ? q[((int64_t)mytok * Hq + myhead) * dim + d] : (bf16_t)0;
+      qf[ks][i] = __builtin_bit_cast(__bf16, w);
+    }
+  }
+  f32x4_t o[NCB];
+#pragma unroll
+  for (int n = 0; n < NCB; ++n) o[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int* bt = tables + (int64_t)seq * W;
+  bf16_t* ph = sPh + wave * 16 * PS;
+  bf16_t* pl = sPl + wave * 16 * PS;
+  const bool vec = (Dr & 7) == 0 && (dim & 7) == 0;
+
+  // decode steps split a row's keys over blockIdx.z: this workgroup takes [kbeg, kend)
+  const int nsplit = gridDim.z;
+  const int kbeg = nsplit > 1 ? blockIdx.z * split_keys : 0;
+  const int kend = nsplit > 1 ? min(maxlen, kbeg + split_keys) : maxlen;
+  constexpr int CPR = (DkP + VP) / 8;             // 16-byte chunks per cache row (padded)
+  constexpr int NCH = (MKT * CPR + NT - 1) / NT;  // chunks per thread
+  const int cpr = (Dr + 7) / 8;                   // chunks that hold data
+  for (int k0 = kbeg; k0 < kend; k0 += MKT) {
+    __syncthreads();  // the previous tile is no longer read (first time: the zero fill is done)
+    // All of a tile's 16-byte chunks are requested before any is used. A tile lies inside one page
+    // when the page size is a multiple of the tile. Consecutive lanes take consecutive keys of one
+    // chunk, so the transposed 2-byte value writes fall into consecutive LDS words.
+    const bool one_page = (bs % MKT) == 0;
+    const int64_t row0 = one_page ? ((int64_t)bt[k0 / bs] * Hkv + g) * bs + (k0 % bs) : 0;
+    u32x4_t pre[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int e = threadIdx.x + i * NT;
+      const int c = e / MKT, j = e - c * MKT;
+      const int key = k0 + j;
+      u32x4_t v = {0, 0, 0, 0};
+      if (c < cpr && key < kend) {
+        const int64_t row = one_page ? row0 + j : ((int64_t)bt[key / bs] * Hkv + g) * bs + (key % bs);
+        const bf16_t* src = cache + row * Dr + c * 8;
+        if (vec) {
+          v = *reinterpret_cast<const u32x4_t*>(src);
+        } else {
+#pragma unroll
+          for (int qq = 0; qq < 8; ++qq)
+            if (c * 8 + qq < Dr) v[qq >> 1] |= (uint32_t)src[qq] << (16 * (qq & 1));
+        }
+      }
+      pre[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int e = threadIdx.x + i * NT;
+      const int c = e / MKT, j = e - c * MKT;
+      if (c >= cpr) continue;
+      if (c * 8 + 8 <= dim) {
+        *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = pre[i];
+      } else {
+#pragma unroll
+        for (int qq = 0; qq < 8; ++qq) {
+          const int d = c * 8 + qq;
+          const bf16_t val = (bf16_t)(pre[i][qq >> 1] >> (16 * (qq & 1)));
+          if (d < dim) sK[j * KS + d] = val;
+          else if (d < Dr) sVt[(d - dim) * VS + j] = val;
+        }
+      }
+    }
+    __syncthreads();
+    // scores of this lane's row against keys k0 + 16 kb + 4 kq + r
+    float sc[2][4];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      f32x4_t a = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(&sK[(kb * 16 + r16) * KS + ks * 32 + kq * 8]);
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], a, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        sc[kb][r] = (k0 + kb * 16 + kq * 4 + r < min(mylen, kend)) ? a[r] * scale : -INFINITY;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sc[kb][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    const float mref = (mn == -INFINITY) ? 0.f : mn;  // a row with no key yet
+    const float corr = expf(m - mref);
+    float psum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float pv = expf(sc[kb][r] - mref);
+        psum += pv;
+        const __bf16 hi = (__bf16)pv;
+        const __bf16 lo = (__bf16)(pv - (float)hi);
+        ph[r16 * PS + kb * 16 + kq * 4 + r] = __builtin_bit_cast(bf16_t, hi);
+        pl[r16 * PS + kb * 16 + kq * 4 + r] = __builtin_bit_cast(bf16_t, lo);
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = mn;
+    // the accumulators hold rows 4 kq + r: their correction comes from the lane that owns the row
+    float cr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, kq * 4 + r, 64);
+    // P is written and read by the same wave only: its own LDS writes are visible after a wave barrier
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    const bf16x8_t pah = *reinterpret_cast<const bf16x8_t*>(&ph[r16 * PS + kq * 8]);
+    const bf16x8_t pal = *reinterpret_cast<const bf16x8_t*>(&pl[r16 * PS + kq * 8]);
+#pragma unroll
+    for (int n = 0; n < NCB; ++n) {
+      const bf16x8_t vb = *reinterpret_cast<const bf16x8_t*>(&sVt[(n * 16 + r16) * VS + kq * 8]);
+      f32x4_t acc = o[n];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[r] *= cr[r];
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pah, vb, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pal, vb, acc, 0, 0, 0);
+      o[n] = acc;
+    }
+  }
+  // o[n][r] = O[row 4 kq + r][column 16 n + r16]
+  if (nsplit > 1) {
+    const int64_t pbase = (((int64_t)blockIdx.x * Hkv + g) * nsplit + blockIdx.z) * 64;
+    if (kq == 0) {
+      part_ml[(pbase + myrow) * 2] = m;
+      part_ml[(pbase + myrow) * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = wave * 16 + kq * 4 + r;
+#pragma unroll
+      for (int n = 0; n < NCB; ++n) {
+        const int col = n * 16 + r16;
+        if (col < vdim) part_o[(pbase + row) * vdim + col] = o[n][r];
+      }
+    }
+    return;
+  }
+  float inv[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) inv[r] = 1.f / __shfl(l, kq * 4 + r, 64);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = wave * 16 + kq * 4 + r;
+    if (row >= ntok * G) continue;
+    const int64_t tok = tok0 + row / G;
+    const int h = g * G + row % G;
+#pragma unroll
+    for (int n = 0; n < NCB; ++n) {
+      const int col = n * 16 + r16;
+      if (col >= vdim) continue;
+      float v = o[n][r] * inv[r];
+      if (gate) v *= 1.f / (1.f + expf(-ld(gate + tok * gate_stride + h * vdim + col)));
+      st(out + (tok * Hq + h) * vdim + col, v);
+    }
+  }
+}
+
+// Merge the key-range partials of a split step: out = sum_z e^(m_z - M) o_z / sum_z e^(m_z - M) l_z.
+__global__ __launch_bounds__(NT) void grouped_attention_merge_kernel(
+    const int* __restrict__ items, int nsplit, const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    int Hq, int Hkv, int vdim, const bf16_t* __restrict__ gate, int64_t gate_stride, bf16_t* __restrict__ out) {
+  const int item = blockIdx.x, g = blockIdx.y, row = blockIdx.z;
+  const int G = Hq / Hkv;
+  const int tok0 = items[item * 3 + 1], ntok = items[item * 3 + 2];
+  if (row >= ntok * G) return;
+  const int64_t base = ((int64_t)item * Hkv + g) * nsplit;
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) M = fmaxf(M, part_ml[((base + z) * 64 + row) * 2]);
+  float L = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float* ml = part_ml + ((base + z) * 64 + row) * 2;
+    L += expf(ml[0] - M) * ml[1];  // an empty range has m = -inf, l = 0
+  }
+  const int64_t tok = tok0 + row / G;
+  const int h = g * G + row % G;
+  for (int c = threadIdx.x; c < vdim; c += NT) {
+    float a = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const int64_t pb = (base + z) * 64 + row;
+      a += expf(part_ml[pb * 2] - M) * part_o[pb * vdim + c];
+    }
+    float v = a / L;
+    if (gate) v *= 1.f / (1.f + expf(-ld(gate + tok * gate_stride + h * vdim + c)));
+    st(out + (tok * Hq + h) * vdim + c, v);
+  }
+}
+
+template <typename T, int VC>
+int launch_attn(const void* q, const void* cache, const int* tables, int W, int bs, const int* row_seq,
+                const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim, int T_rows, int QT,
+                const void* gate, int64_t gate_stride, void* out, hipStream_t stream) {
+  const int Dr = dim + vdim;
+  int KT = 64;
+  while (KT > 16 && ((size_t)KT * (Dr + 1) + (size_t)QT * 4 * dim) * 4 > 128 * 1024) KT >>= 1;
+  const size_t lds = ((size_t)KT * (Dr + 1) + (size_t)QT * 4 * dim) * 4;
+  if (lds > 160 * 1024) return 1;
+  const int G = Hq / Hkv;
+  const dim3 grid((T_rows + QT - 1) / QT, Hkv * ((G + 3) / 4));
+  auto go = [&](auto kern) {
+    if (lds > 64 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(kern, grid, dim3(NT), lds, stream, (const T*)q, (const T*)cache, tables, W, bs, row_seq, row_len,
+                       scale, Hq, Hkv, dim, vdim, KT, T_rows, (const T*)gate, gate_stride, (T*)out);
+  };
+  if (QT == 4) go(grouped_attention_kernel<T, VC, 4>);
+  else go(grouped_attention_kernel<T, VC, 1>);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const int64_t* positions,
+                       const float* cos_sin, int Hq, int Hkv, int dim, int vdim, int rot_dims, int interleaved,
+                       int unit, float eps, float* v_first, int v_mode, float lam, const int64_t* slots, void* cache,
+                       int bs, void* q_out, int T, int f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    hipLaunchKernelGGL((qkv_rope_cache_kernel<float>), dim3(T), dim3(NT), 0, stream, (const float*)qkv, stride, bias,
+                       positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
+                       slots, (float*)cache, bs, (float*)q_out);
+  else
+    hipLaunchKernelGGL((qkv_rope_cache_kernel<bf16_t>), dim3(T), dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias,
+                       positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
+                       slots, (bf16_t*)cache, bs, (bf16_t*)q_out);
+}
+
+// Returns 0, or 1 when the sizes do not fit the kernel (vdim > 1024 or rows too wide for LDS).
+int sm_grouped_attention(const void* q, const void* cache, const int* tables, int W, int bs, const int* row_seq,
+                         const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim, int T, int QT,
+                         const void* gate, int64_t gate_stride, void* out, int f32, hipStream_t stream) {
+  if (T == 0) return 0;
+  const int vc = (vdim + 63) / 64;
+#define SM_GO(TYPE, VC)                                                                                          \
+  return launch_attn<TYPE, VC>(q, cache, tables, W, bs, row_seq, row_len, scale, Hq, Hkv, dim, vdim, T, QT, gate, \
+                               gate_stride, out, stream)
+  if (f32) {
+    if (vc <= 1) SM_GO(float, 1);
+    if (vc <= 2) SM_GO(float, 2);
+    if (vc <= 4) SM_GO(float, 4);
+    if (vc <= 8) SM_GO(float, 8);
+    if (vc <= 16) SM_GO(float, 16);
+  } else {
+    if (vc <= 1) SM_GO(bf16_t, 1);
+    if (vc <= 2) SM_GO(bf16_t, 2);
+    if (vc <= 4) SM_GO(bf16_t, 4);
+    if (vc <= 8) SM_GO(bf16_t, 8);
+    if (vc <= 16) SM_GO(bf16_t, 16);
+  }
+#undef SM_GO
+  return 1;
+}
+
+// bf16, matrix cores. Returns 0, or 1 when the sizes are outside the compiled forms
+// (dim > 256, vdim > 256, group size > 64).
+int sm_grouped_attention_mfma(const void* q, const void* cache, const int* tables, int W, int bs, const int* items,
+                              int n_items, const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim,
+                              const void* gate, int64_t gate_stride, void* out, int nsplit, int split_keys,
+                              float* part_o, float* part_ml, hipStream_t stream) {
+  if (n_items == 0) return 0;
+  const int nks = (dim + 31) / 32, ncb = (vdim + 15) / 16;
+  if (Hq / Hkv > 64 || nks > 8 || ncb > 16) return 1;
+  const dim3 grid(n_items, Hkv, nsplit);
+#define SM_GO(NKS, NCB)                                                                                           \
+  hipLaunchKernelGGL((grouped_attention_mfma_kernel<NKS, NCB>), grid, dim3(NT), 0, stream, (const bf16_t*)q,       \
+                     (const bf16_t*)cache, tables, W, bs, items, row_len, scale, Hq, Hkv, dim, vdim,               \
+                     (const bf16_t*)gate, gate_stride, (bf16_t*)out, split_keys, part_o, part_ml)
+  if (nks <= 2 && ncb <= 4) SM_GO(2, 4);
+  else if (nks <= 4 && ncb <= 8) SM_GO(4, 8);
+  else SM_GO(8, 16);
+#undef SM_GO
+  if (nsplit > 1)
+    hipLaunchKernelGGL(grouped_attention_merge_kernel, dim3(n_items, Hkv, 64), dim3(NT), 0, stream, items, nsplit,
+                       part_o, part_ml, Hq, Hkv, vdim, (const bf16_t*)gate, gate_stride, (bf16_t*)out);
+  return 0;
+}
+
+}  // extern "C"
