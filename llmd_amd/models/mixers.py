@@ -281,6 +281,8 @@ class GroupedAttention(torch.nn.Module):
         if self.v_mix:
             v_first = shared.get("v_first")
             mode = 2 if v_first is not None else 1
+            if v_first is not None and v_first.shape[1] != self.nv:
+                raise ValueError("value mixing needs the same kv heads x value size in all layers that use it")
             if v_first is None:
                 v_first = shared["v_first"] = torch.empty(T, self.nv, dtype=torch.float32, device=h.device)
         sm.qkv_rope_cache(p, self.bias32, meta.positions, self.cos_sin, self.Hq, self.Hkv, self.dim, self.vdim,

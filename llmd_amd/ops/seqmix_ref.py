@@ -232,7 +232,7 @@ def _act(z, kind):
 
 
 def gated_act(gu, Fh, kind):
-    return (_act(gu[:, :Fh].float(), kind) * gu[:, Fh:].float()).to(gu.dtype)
+    return (_act(gu[:, :Fh].float(), kind) * gu[:, Fh:2 * Fh].float()).to(gu.dtype)
 
 
 def moe_route_scores(logits, correction, k):

@@ -185,3 +185,51 @@ def forward(cfg, w, tokens):
         per_layer.append(sum(streams))
     x = layer_norm(sum(streams), w["final.norm"], eps)
     return x @ w["head"].to(F64).T, torch.stack(per_layer)
+
+
+def random_weights(cfg, seed=0):
+    """Random bfloat16 tensors with the checkpoint's names and shapes. Nothing is left at a value
+    that would hide a mechanism: stream mixes are far from the identity, biases and corrections
+    are of the size of what they are added to, norm weights differ from 1."""
+    g = torch.Generator().manual_seed(seed)
+    d, V, S = cfg["width"], cfg["vocab"], cfg.get("streams")
+    w = {}
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean).to(torch.bfloat16)
+
+    def lin(o, i):
+        return rnd(o, i, std=1.0 / math.sqrt(i))
+
+    w["embed"] = rnd(V, d)
+    w["final.norm"] = rnd(d, std=0.2, mean=1.0)
+    w["head"] = lin(V, d)
+    for i, spec in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", spec["mixer"]
+        H, G, dim, vdim = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        for q in (1, 2) if spec.get("mlp") else (1,):
+            w[f"{p}norm{q}"] = rnd(d, std=0.2, mean=1.0)
+            if S:
+                w[f"{p}hc{q}.in"] = rnd(S, std=0.5, mean=0.6)
+                w[f"{p}hc{q}.out"] = rnd(S, std=0.5, mean=0.7)
+                w[f"{p}hc{q}.mix"] = (torch.eye(S) * 0.8 + torch.randn(S, S, generator=g) * 0.3).to(torch.bfloat16)
+        w[p + "mix.q"], w[p + "mix.q.b"] = lin(H * dim, d), rnd(H * dim, std=0.5)
+        w[p + "mix.k"], w[p + "mix.k.b"] = lin(G * dim, d), rnd(G * dim, std=0.5)
+        w[p + "mix.v"], w[p + "mix.v.b"] = lin(G * vdim, d), rnd(G * vdim, std=0.5)
+        w[p + "mix.vmix"] = torch.tensor(0.2 + 0.6 * torch.rand((), generator=g).item()).to(torch.bfloat16)
+        w[p + "mix.g"] = lin(H * vdim, d)
+        w[p + "mix.o"] = lin(d, H * vdim)
+        f = spec.get("mlp")
+        if not f:
+            continue
+        if f["kind"] == "dense":
+            w[p + "mlp.gate"], w[p + "mlp.up"], w[p + "mlp.down"] = lin(f["ff"], d), lin(f["ff"], d), lin(d, f["ff"])
+        else:
+            r, ff = f["router"], f["expert"]["ff"]
+            n = r["experts"] + r.get("identity", 0)
+            w[p + "mlp.router"] = rnd(n, d, std=2.0 / math.sqrt(d))
+            w[p + "mlp.correction"] = rnd(n, std=0.3)
+            for e in range(r["experts"]):
+                w[f"{p}mlp.e{e}.gate"], w[f"{p}mlp.e{e}.up"] = lin(ff, d), lin(ff, d)
+                w[f"{p}mlp.e{e}.down"] = lin(d, ff)
+    return w

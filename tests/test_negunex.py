@@ -1,0 +1,585 @@
+"""Negunex on the engine against the plain float64 oracle (tests/negunex_oracle.py): every
+mechanism alone, whole prompts against token-by-token decoding and portions down to two tokens,
+mixed batches of unequal requests over pages that are freed and reused, keys far away and on
+either side of page borders and of a row's last visible key, the first token, long decoding,
+other sizes, greedy generation through the scheduler. Each case runs on the CPU reference ops
+and, marked gpu, on the HIP kernels."""
+import json
+import math
+import os
+
+import pytest
+import torch
+from safetensors.torch import save_file
+
+import negunex_oracle as oracle
+from llmd_amd.engine.config import EngineConfig, ModelConfig
+from llmd_amd.engine.engine import LLMEngine
+from llmd_amd.engine.request import SamplingParams
+from llmd_amd.ops import seqmix as sm
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+F64 = torch.float64
+
+
+def attn(heads, kv, dim, vdim, scale=None, rot_dims=None, base=10000.0, scaling=None, v_mix=False):
+    rot = None if rot_dims == 0 else {"dims": rot_dims or dim, "base": base}
+    if rot and scaling:
+        rot["scaling"] = scaling
+    m = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": scale or 1.0 / math.sqrt(dim),
+         "v_mix": v_mix}
+    if rot:
+        m["rot"] = rot
+    return {"type": "attention", "mixer": m}
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(ff, experts, top, identity=0):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "identity": identity, "top": top}}
+
+
+def config(layers, width=48, vocab=70, streams=2, eps=1e-5):
+    c = {"architecture": "Negunex", "width": width, "vocab": vocab, "norm": {"eps": eps},
+         "layers": [dict(l, mlp=f) for l, f in layers]}
+    if streams is not None:
+        c["streams"] = streams
+    return c
+
+
+SCALING = {"factor": 3.0, "low": 1.0, "high": 3.0, "original": 48}  # positions beyond 48 feel it
+# sizes that differ wherever the design lets them: key != value size, partial rotary, scaled
+# frequencies, three streams, value mixing that starts at the second layer, identity experts,
+# a layer without feed-forward, two attention geometries
+MIXED = config([(attn(6, 3, 24, 40, scale=0.4, rot_dims=16, base=300.0, scaling=SCALING), dense(72)),
+                (attn(6, 3, 24, 40, scale=0.3, rot_dims=24, base=50.0, v_mix=True), moe(24, 5, 2, identity=2)),
+                (attn(3, 3, 16, 40, scale=0.5, rot_dims=8, v_mix=True), None),
+                (attn(6, 3, 32, 40, scale=0.2, rot_dims=32, scaling=SCALING, v_mix=True), moe(40, 3, 1, identity=1))],
+               width=48, vocab=70, streams=3)
+# values the first configuration keeps apart, made equal or 1 here; no streams at all
+PLAIN = config([(attn(1, 1, 16, 16, scale=1.0, rot_dims=16, v_mix=True), moe(16, 4, 4)),
+                (attn(4, 1, 16, 16, rot_dims=0, v_mix=True), dense(64)),
+                (attn(2, 1, 32, 32, rot_dims=2), moe(8, 1, 1, identity=1))], width=32, vocab=64, streams=None)
+ONE_STREAM = config([(attn(2, 2, 16, 8, v_mix=True), dense(40)), (attn(4, 2, 16, 8, v_mix=True), moe(16, 2, 2, 2))],
+                    width=32, vocab=40, streams=1)
+# multiples of nothing: vector loads, matrix-core padding and lane groups all take their slow paths
+ODD = config([(attn(9, 3, 10, 14, scale=0.7, rot_dims=6, base=77.0, scaling=SCALING, v_mix=True), moe(22, 7, 3, 2)),
+              (attn(5, 5, 18, 6, rot_dims=10), dense(26)),
+              (attn(9, 3, 6, 14, scale=0.9, rot_dims=2, v_mix=True), None)], width=34, vocab=51, streams=4, eps=1e-4)
+
+
+def model_dir(tmp_path, cfg, seed=0):
+    W = oracle.random_weights(cfg, seed)
+    d = tmp_path / f"m{seed}"
+    d.mkdir(exist_ok=True)
+    (d / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in W.items()}, str(d / "model.safetensors"))
+    return str(d), W
+
+
+def engine(path, device, dtype="float32", pages=16, seqs=4, **kw):
+    mc = ModelConfig.from_hf(path)
+    kw.setdefault("enable_prefix_caching", False)
+    cfg = EngineConfig.create(path, model_config=mc, device=device, dtype=dtype, load_format="safetensors",
+                              weights_path=path, block_size=64, num_gpu_blocks=pages, max_num_seqs=seqs,
+                              max_model_len=pages * 64 + 1, max_num_batched_tokens=pages * 64,
+                              enforce_eager=True, prefill_token_align=0, **kw)
+    return LLMEngine(cfg, capture_graphs=False)
+
+
+def row_errs(got, want):
+    d = got.double().cpu() - want
+    return torch.sqrt((d * d).mean(-1)) / torch.sqrt((want * want).mean())
+
+
+def rel_err(got, want):
+    return float(row_errs(got, want).max())
+
+
+def close(got, want, dtype):
+    """float32: every row within rounding of the oracle. bfloat16: the rounding of the router's
+    input can flip a close choice of experts in a row, so nine rows in ten are held to the bound."""
+    e = row_errs(got, want)
+    if dtype == "float32":
+        return float(e.max()) < 2e-4
+    return float(e.quantile(0.9)) < 6e-2 and float(e.median()) < 3e-2
+
+
+def replay(eng, prompts, steps):
+    """steps: list of lists of (name, count). Returns name -> logits [len, vocab] (all positions)."""
+    at = {n: 0 for n in prompts}
+    out = {n: [] for n in prompts}
+    for step in steps:
+        entries, end = [], []
+        for n, c in step:
+            toks = prompts[n][at[n]:at[n] + c]
+            entries.append((n, toks, list(range(len(toks)))))
+            at[n] += c
+            if at[n] == len(prompts[n]):
+                end.append(n)
+        lg = eng.forced_step(entries, end)
+        o = 0
+        for n, c in step:
+            out[n].append(lg[o:o + c].cpu())
+            o += c
+    return {n: torch.cat(v) for n, v in out.items() if v}
+
+
+def tokens(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+# ------------------------------------------------------------------ mechanisms alone (ops)
+def _dev(t, device, dtype=None):
+    return (t if dtype is None else t.to(dtype)).to(device)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("S,d", [(1, 40), (2, 33), (5, 300)])
+def test_streams_and_layer_norm(device, S, d):
+    g = torch.Generator().manual_seed(S)
+    T = 7
+    x0 = torch.randn(T, d, generator=g) + 3.0   # a mean far from zero: a one-pass variance would show
+    streams = [x0 * (s + 1) for s in range(S)]
+    w_in, w_out = torch.randn(S, generator=g), torch.randn(S, generator=g)
+    mix, nxt = torch.randn(S, S, generator=g), torch.randn(S, generator=g)
+    nw, nw2 = torch.randn(d, generator=g), torch.randn(d, generator=g)
+    y = torch.randn(T, d, generator=g)
+    X = _dev(torch.stack(streams), device)
+    h = sm.hyper_norm(X, _dev(w_in, device), _dev(nw, device), 1e-5, torch.float32)
+    assert rel_err(h, oracle.layer_norm(oracle.hyper_in(streams, w_in), nw, 1e-5)) < 1e-5
+    h2 = sm.hyper_update_norm(X, _dev(y, device), _dev(mix, device), _dev(w_out, device), _dev(nxt, device),
+                              _dev(nw2, device), 1e-5, torch.float32)
+    new = oracle.hyper_out([s.double() for s in streams], y.double(), mix, w_out)
+    assert rel_err(X, torch.stack(new)) < 1e-5
+    assert rel_err(h2, oracle.layer_norm(oracle.hyper_in(new, nxt), nw2, 1e-5)) < 1e-5
+    # without a following norm only the streams move
+    X2 = _dev(torch.stack(streams), device)
+    assert sm.hyper_update_norm(X2, _dev(y, device), _dev(mix, device), _dev(w_out, device)) is None
+    assert rel_err(X2, torch.stack(new)) < 1e-5
+
+
+def test_frequency_scaling_table():
+    from llmd_amd.models.mixers import rope_table
+
+    for dims, base, sc in [(16, 300.0, SCALING), (6, 77.0, SCALING), (8, 10000.0, None),
+                           (32, 5e5, {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192})]:
+        f = oracle.rotary_frequencies(dims, base, sc)
+        if sc is SCALING and dims == 16:  # all three branches occur
+            plain = oracle.rotary_frequencies(dims, base)
+            ratios = [a / b for a, b in zip(f, plain)]
+            assert ratios[0] == 1.0 and abs(ratios[-1] - 1 / 3) < 1e-12 and any(1 / 3 < r < 1 for r in ratios)
+        tab = rope_table(dims, base, 200, "cpu", sc)
+        want = torch.tensor([[math.cos(p * x) for x in f] + [math.sin(p * x) for x in f] for p in (0, 1, 57, 199)],
+                            dtype=F64)
+        assert torch.allclose(tab[[0, 1, 57, 199]].double(), want, atol=1e-6)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("Hq,Hkv,dim,vdim,rot", [(6, 3, 24, 40, 16), (2, 2, 10, 6, 10), (4, 1, 130, 20, 64),
+                                                  (3, 3, 8, 8, 0)])
+def test_projection_rotary_norm_cache(device, interleaved, Hq, Hkv, dim, vdim, rot):
+    from llmd_amd.models.mixers import rope_table
+
+    g = torch.Generator().manual_seed(dim)
+    T, bs, eps = 9, 64, 1e-5
+    n = (Hq + Hkv) * dim + Hkv * vdim
+    qkv, bias = torch.randn(T, n + 5, generator=g), torch.randn(n, generator=g)
+    pos = torch.tensor([0, 1, 2, 63, 64, 65, 150, 199, 3])
+    slots = torch.tensor([5, 64 + 1, 2, 63, 128, 190, -1, 0, 64])
+    tab = rope_table(rot, 50.0, 200, "cpu", SCALING) if rot else None
+    vf = torch.randn(T, Hkv * vdim, generator=g)
+    for mode, lam in ((0, 0.0), (1, 0.0), (2, 0.3)):
+        cache = torch.zeros(3, Hkv, bs, dim + vdim)
+        q_out = torch.zeros(T, Hq, dim)
+        vbuf = vf.clone()
+        cache_d, q_d, v_d = _dev(cache, device), _dev(q_out, device), _dev(vbuf, device)
+        sm.qkv_rope_cache(_dev(qkv, device), _dev(bias, device), _dev(pos, device), _dev(tab, device) if rot else None,
+                          Hq, Hkv, dim, vdim, rot, interleaved, eps, v_d if mode else None, mode, lam,
+                          _dev(slots, device), cache_d, q_d)
+        x = qkv[:, :n].double() + bias.double()
+        q = x[:, :Hq * dim].view(T, Hq, dim)
+        k = x[:, Hq * dim:(Hq + Hkv) * dim].view(T, Hkv, dim)
+        v = x[:, (Hq + Hkv) * dim:].view(T, Hkv, vdim)
+        if rot:
+            if interleaved:
+                q = oracle.rotate_interleaved(q, pos.tolist(), rot, 50.0, SCALING)
+                k = oracle.rotate_interleaved(k, pos.tolist(), rot, 50.0, SCALING)
+            else:
+                f = torch.tensor(oracle.rotary_frequencies(rot, 50.0, SCALING), dtype=F64)
+                a = pos.double()[:, None, None] * f
+                def half(t):
+                    u, w = t[..., :rot // 2], t[..., rot // 2:rot]
+                    return torch.cat([u * a.cos() - w * a.sin(), w * a.cos() + u * a.sin(), t[..., rot:]], -1)
+                q, k = half(q), half(k)
+        q, k = oracle.unit_rms(q, eps), oracle.unit_rms(k, eps)
+        if mode == 1:
+            assert rel_err(v_d, v.reshape(T, -1)) < 1e-6
+        if mode == 2:
+            v = (1 - lam) * v + lam * vf.double().view(T, Hkv, vdim)
+        assert rel_err(q_d, q) < 1e-5
+        got = cache_d.cpu()
+        for t in range(T):
+            s = int(slots[t])
+            if s < 0:
+                continue
+            row = got[s // bs, :, s % bs].double()
+            assert torch.allclose(row[:, :dim], k[t], atol=1e-5) and torch.allclose(row[:, dim:], v[t], atol=1e-5), t
+        written = {int(s) for s in slots if s >= 0}
+        mask = torch.ones(3 * bs, dtype=torch.bool)
+        mask[list(written)] = False
+        assert float(got.permute(0, 2, 1, 3).reshape(3 * bs, -1)[mask].abs().max()) == 0.0  # nothing else is touched
+
+
+def _paged(rows, bs, device, dtype, seed=1):
+    """rows [n, Hkv, Dr] scattered over shuffled pages of a cache filled with noise; (cache, table row)."""
+    n, Hkv, Dr = rows.shape
+    nb = -(-n // bs)
+    perm = torch.randperm(nb + 3, generator=torch.Generator().manual_seed(seed))[:nb]
+    cache = torch.randn(nb + 3, Hkv, bs, Dr, generator=torch.Generator().manual_seed(seed + 1)).to(dtype)
+    for i in range(n):
+        cache[perm[i // bs], :, i % bs] = rows[i].to(dtype)
+    return cache.to(device), perm.int()
+
+
+def _seq_meta(device, tables, q_lens, lens):
+    """SeqMeta of a step: sequence i brings q_lens[i] tokens that end at context length lens[i]."""
+    from llmd_amd.engine.attn_meta import SeqMeta
+
+    n = len(q_lens)
+    start = [0]
+    for c in q_lens:
+        start.append(start[-1] + c)
+    row_seq = [i for i, c in enumerate(q_lens) for _ in range(c)]
+    row_len = [lens[i] - c + j + 1 for i, c in enumerate(q_lens) for j in range(c)]
+    W = max(len(t) for t in tables)
+    tab = torch.zeros(n, W, dtype=torch.int32)
+    for i, t in enumerate(tables):
+        tab[i, :len(t)] = t
+    ti = lambda v: torch.tensor(v, dtype=torch.int32, device=device)  # noqa: E731
+    return SeqMeta(n, ti(start), ti([0] * n), ti([0] * n), ti(row_seq), ti(row_len), tab.to(device),
+                   max_len=max(lens), max_q=max(q_lens), q_lens=list(q_lens))
+
+
+def _attention_oracle(q, rows, dim, row_len, scale, gate):
+    """q [T, Hq, dim] against rows [n, Hkv, dim + vdim] of ONE sequence, row t seeing row_len[t] keys."""
+    T, Hq, _ = q.shape
+    Hkv = rows.shape[1]
+    out = torch.zeros(T, Hq, rows.shape[2] - dim, dtype=F64)
+    for t in range(T):
+        for h in range(Hq):
+            kv = rows[:row_len[t], h // (Hq // Hkv)].double()
+            p = torch.softmax((kv[:, :dim] @ q[t, h].double()) * scale, 0)
+            out[t, h] = p @ kv[:, dim:]
+    out = out.reshape(T, -1)
+    return out if gate is None else out * torch.sigmoid(gate.double())
+
+
+ATT_DTYPES = [("cpu", torch.float32), pytest.param("cuda", torch.float32, marks=pytest.mark.gpu),
+              pytest.param("cuda", torch.bfloat16, marks=pytest.mark.gpu)]
+
+
+@pytest.mark.parametrize("device,dtype", ATT_DTYPES)
+@pytest.mark.parametrize("decode", [False, True], ids=["prompt", "decoded"])
+@pytest.mark.parametrize("where", ["far", "page-end", "page-start", "last-seen", "first-unseen"])
+def test_one_key_stands_out(device, dtype, where, decode):
+    """One key among 300 has a score far above the rest: the output is its value if and only if the
+    row may see it - far back, on either side of a page border, the last visible key, and the first
+    one beyond the row's length; as the last row of a 5-token portion and as a single decoded token."""
+    Hq, Hkv, dim, vdim, n, seen = 6, 3, 24, 40, 300, 200
+    g = torch.Generator().manual_seed(7)
+    rows = torch.randn(n, Hkv, dim + vdim, generator=g) * 0.3
+    nq = 1 if decode else 5
+    q = torch.randn(nq, Hq, dim, generator=g) * 0.3
+    j = {"far": 2, "page-end": 63, "page-start": 64, "last-seen": seen - 1, "first-unseen": seen}[where]
+    h = 3                                                  # query head 3 reads kv head 1
+    rows[j, 1, :dim] = q[-1, h] / q[-1, h].norm() * 12.0   # and looks straight at key j
+    q[-1, h] *= 6.0
+    rows, q = rows.to(dtype).float(), q.to(dtype).float()  # the values both sides compute with
+    cache, table = _paged(rows, 64, device, dtype)
+    seq = _seq_meta(device, [table], [nq], [seen])
+    gate = torch.randn(nq, Hq * vdim, generator=g).to(dtype)
+    out = sm.grouped_attention(q.to(dtype).to(device), cache, dim, vdim, 1.0, seq, gate.to(device))
+    lens = [seen - nq + i + 1 for i in range(nq)]
+    want = _attention_oracle(q, rows, dim, lens, 1.0, gate.float())
+    assert rel_err(out.float(), want) < (1e-4 if dtype == torch.float32 else 2e-2)
+    ungated = sm.grouped_attention(q.to(dtype).to(device), cache, dim, vdim, 1.0, seq, None)
+    hit = torch.allclose(ungated[-1].float().cpu().view(Hq, vdim)[h], rows[j, 1, dim:], atol=2e-2)
+    assert hit == (where != "first-unseen")
+
+
+@pytest.mark.parametrize("device,dtype", ATT_DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,dim,vdim", [(6, 3, 24, 40), (5, 5, 10, 14), (8, 1, 64, 128), (2, 2, 130, 20),
+                                             (4, 2, 256, 256), (70, 1, 8, 8)])
+@pytest.mark.parametrize("decode_only", [False, True], ids=["mixed-step", "decode-step"])
+def test_grouped_attention_steps(device, dtype, Hq, Hkv, dim, vdim, decode_only):
+    """Several sequences of unequal length in one step, pages shuffled: single decoded tokens (one far
+    beyond 256 keys, which cuts the keys into ranges on the matrix cores) beside prompt portions that
+    start at 0, in mid-page and at a page border."""
+    g = torch.Generator().manual_seed(Hq * dim)
+    lens = [700, 65, 1] if decode_only else [300, 64, 130, 7, 1]
+    q_lens = [1, 1, 1] if decode_only else [1, 1, 66, 7, 1]
+    caches, tables, off = [], [], 0
+    all_rows = [torch.randn(n, Hkv, dim + vdim, generator=g).to(dtype).float() for n in lens]
+    total = sum(-(-n // 64) for n in lens) + 2
+    cache = torch.randn(total, Hkv, 64, dim + vdim, generator=g).to(dtype)
+    perm = torch.randperm(total, generator=g).int()
+    for rows in all_rows:
+        nb = -(-rows.shape[0] // 64)
+        tab = perm[off:off + nb]
+        off += nb
+        for i in range(rows.shape[0]):
+            cache[tab[i // 64], :, i % 64] = rows[i].to(dtype)
+        tables.append(tab)
+    seq = _seq_meta(device, tables, q_lens, lens)
+    T = sum(q_lens)
+    q = (torch.randn(T, Hq, dim, generator=g) * 0.5).to(dtype)
+    gate = torch.randn(T, Hq * vdim + 8, generator=g).to(dtype)[:, 3:3 + Hq * vdim]  # a strided column view
+    out = sm.grouped_attention(q.to(device), cache.to(device), dim, vdim, 0.3, seq, gate.to(device))
+    t0 = 0
+    for rows, c, n in zip(all_rows, q_lens, lens):
+        want = _attention_oracle(q[t0:t0 + c].float(), rows, dim, [n - c + i + 1 for i in range(c)], 0.3,
+                                 gate[t0:t0 + c].float())
+        assert rel_err(out[t0:t0 + c].float(), want) < (1e-4 if dtype == torch.float32 else 2e-2)
+        t0 += c
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("E,I,k", [(5, 2, 2), (3, 0, 1), (4, 4, 8), (1, 1, 1), (130, 6, 8), (600, 3, 3)])
+def test_score_router(device, E, I, k):
+    g = torch.Generator().manual_seed(E)
+    T, d = 50, 24
+    h, router = torch.randn(T, d, generator=g), torch.randn(E + I, d, generator=g) * 0.5
+    corr = torch.randn(E + I, generator=g) * 0.5    # large enough to change most choices
+    ids, ws = oracle.route(h, router, corr, k)
+    plain, _ = oracle.route(h, router, torch.zeros(E + I), k)
+    if E + I > k:
+        assert (ids.sort(-1).values != plain.sort(-1).values).any()
+    logits = (h.double() @ router.double().T).float()
+    gi, gw = sm.moe_route_scores(_dev(logits, device), _dev(corr, device), k)
+    order = gi.cpu().long().sort(-1)
+    want = ids.sort(-1)
+    assert torch.equal(order.values, want.values)
+    assert torch.allclose(torch.gather(gw.cpu().double(), 1, order.indices), torch.gather(ws, 1, want.indices),
+                          atol=1e-6)
+    assert torch.allclose(gw.sum(-1).cpu(), torch.ones(T), atol=1e-5)
+
+
+@pytest.mark.parametrize("device,dtype", ATT_DTYPES)
+@pytest.mark.parametrize("T,d,F,E,I,k", [(70, 48, 24, 5, 2, 2), (300, 256, 200, 16, 0, 3), (9, 64, 72, 4, 4, 4),
+                                         (33, 50, 30, 3, 1, 1), (700, 64, 136, 2, 1, 2)])
+def test_gated_experts_with_identity(device, dtype, T, d, F, E, I, k):
+    g = torch.Generator().manual_seed(T)
+    h = torch.randn(T, d, generator=g).to(dtype)
+    w1 = (torch.randn(E, 2 * F, d, generator=g) / math.sqrt(d)).to(dtype)
+    w2 = (torch.randn(E, d, F, generator=g) / math.sqrt(F)).to(dtype)
+    ids = torch.stack([torch.randperm(E + I, generator=g)[:k] for _ in range(T)]).int()
+    ws = torch.rand(T, k, generator=g)
+    got = sm.moe_gated_ffn(h.to(device), ids.to(device), ws.to(device), w1.to(device), w2.to(device), "silu")
+    want = torch.zeros(T, d, dtype=F64)
+    hd = h.double()
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            if e >= E:
+                y = hd[t]
+            else:
+                gu = w1[e].double() @ hd[t]
+                y = w2[e].double() @ (oracle.silu(gu[:F]) * gu[F:])
+            want[t] += ws[t, j].double() * y
+    assert rel_err(got.float(), want) < (1e-4 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("kind", ["gelu_tanh", "silu"])
+def test_gated_activation(device, kind):
+    g = torch.Generator().manual_seed(3)
+    gu = torch.randn(11, 2 * 37 + 3, generator=g) * 3
+    got = sm.gated_act(_dev(gu, device), 37, kind)
+    act = oracle.gelu_tanh if kind == "gelu_tanh" else oracle.silu
+    assert rel_err(got, act(gu[:, :37].double()) * gu[:, 37:74].double()) < 1e-5
+
+
+# ------------------------------------------------------------------ the model on the engine
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("layer,streams", [((attn(6, 3, 24, 40, rot_dims=16, scaling=SCALING), dense(72)), 2),
+                                           ((attn(4, 2, 16, 8, scale=0.6), moe(24, 5, 2, identity=2)), 3),
+                                           ((attn(3, 1, 16, 24, rot_dims=0), None), 2),
+                                           ((attn(2, 2, 16, 16), dense(20)), None),
+                                           ((attn(2, 2, 16, 16, v_mix=True), moe(8, 3, 3)), 1)],
+                         ids=["attention+dense", "attention+experts", "attention-only", "no-streams", "one-stream"])
+def test_each_layer_kind_alone(tmp_path, device, layer, streams):
+    cfg = config([layer], streams=streams)
+    path, W = model_dir(tmp_path, cfg)
+    toks = tokens(70, cfg["vocab"], 1)
+    want, _ = oracle.forward(cfg, W, toks)
+    got = replay(engine(path, device), {"a": toks}, [[("a", 70)]])["a"]
+    assert rel_err(got, want) < 2e-4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_layer_streams(tmp_path, device):
+    """The sum of the streams after every layer, not only the logits."""
+    import numpy as np
+
+    path, W = model_dir(tmp_path, MIXED)
+    toks = tokens(40, MIXED["vocab"], 2)
+    _, per_layer = oracle.forward(MIXED, W, toks)
+    r = engine(path, device).runner
+    pl = {"graph": False, "nd": 0, "ids": toks, "pos": list(range(40)), "slots": list(range(40)),
+          "d_bt": np.zeros((0, r.width), "int32"), "d_len": np.zeros(0, "int32"), "p_ql": [40], "p_ctx": [40],
+          "p_bt": np.zeros((1, r.width), "int32"), "rows": [], "seq": ([0], [0])}
+    ids, meta = r._eager_meta(pl)
+    got = []
+    r.model(ids, meta, layer_out=got)
+    assert len(got) == len(MIXED["layers"])
+    for i, (a, b) in enumerate(zip(got, per_layer)):
+        assert rel_err(a, b) < 1e-4, i
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_decode_and_portions_agree(tmp_path, device, dtype):
+    path, W = model_dir(tmp_path, MIXED)
+    toks = tokens(150, MIXED["vocab"], 3)
+    want, _ = oracle.forward(MIXED, W, toks)
+    whole = replay(engine(path, device, dtype), {"a": toks}, [[("a", 150)]])["a"]
+    assert close(whole, want, dtype)
+    # a short prompt, then 140 tokens one by one over two page borders
+    dec = replay(engine(path, device, dtype), {"a": toks}, [[("a", 10)]] + [[("a", 1)]] * 140)["a"]
+    assert close(dec, want, dtype)
+    # portions that end just before, at and just after the page borders, down to two and one tokens
+    cuts = [2, 61, 1, 3, 2, 58, 1, 1, 2, 19]
+    assert sum(cuts) == 150
+    por = replay(engine(path, device, dtype), {"a": toks}, [[("a", c)] for c in cuts])["a"]
+    assert close(por, want, dtype)
+    if dtype == "float32":  # the three ways differ by rounding only
+        assert rel_err(dec, whole.double()) < 1e-4 and rel_err(por, whole.double()) < 1e-4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_mixed_batches_reuse_pages(tmp_path, device):
+    """Five unequal requests through three live places and seven pages: portions beside single
+    tokens, requests that pause, end and hand their pages to the next one."""
+    path, W = model_dir(tmp_path, MIXED)
+    lens = {"a": 130, "b": 1, "c": 67, "d": 90, "e": 64}
+    prompts = {n: tokens(k, MIXED["vocab"], 10 + i) for i, (n, k) in enumerate(lens.items())}
+    steps = [[("a", 60), ("b", 1), ("c", 2)],
+             [("c", 1), ("a", 4)],
+             [("a", 1), ("c", 62), ("d", 30)],           # b's page reused by d
+             [("d", 1), ("a", 63)],                      # a reaches 128: exactly two pages
+             [("c", 1), ("d", 34), ("a", 1)],
+             [("c", 1), ("a", 1), ("d", 25)],            # all three end: every page is free again
+             [("e", 3)],
+             [("e", 61)],
+             ]
+    eng = engine(path, device, pages=7, seqs=3)
+    got = replay(eng, prompts, steps)
+    for n in prompts:
+        assert got[n].shape[0] == lens[n], n
+        assert rel_err(got[n], oracle.forward(MIXED, W, prompts[n])[0]) < 2e-4, n
+    eng.bm.check_invariants()
+    assert eng.bm.num_free() == 7
+    # each alone gives the same rows up to rounding
+    alone = replay(engine(path, device, pages=6, seqs=3), {"d": prompts["d"]}, [[("d", 90)]])["d"]
+    assert rel_err(got["d"], alone.double()) < 1e-4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cfg", [PLAIN, ONE_STREAM, ODD], ids=["equal-or-one", "one-stream", "odd"])
+def test_other_sizes(tmp_path, device, cfg, dtype):
+    path, W = model_dir(tmp_path, cfg, seed=5)
+    toks = tokens(80, cfg["vocab"], 6)
+    want, _ = oracle.forward(cfg, W, toks)
+    got = replay(engine(path, device, dtype), {"a": toks},
+                 [[("a", 5)], [("a", 60)], [("a", 2)]] + [[("a", 1)]] * 13)["a"]
+    assert close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_value_mixing_reaches_the_logits(tmp_path, device):
+    """The same weights with the mixing weight of one later layer changed give other logits, and the
+    first value-mixing layer's own weight changes nothing."""
+    path, W = model_dir(tmp_path, MIXED, seed=9)
+    toks = tokens(30, MIXED["vocab"], 4)
+    base = replay(engine(path, device), {"a": toks}, [[("a", 30)]])["a"]
+
+    def with_vmix(layer, val, sub):
+        W2 = dict(W)
+        W2[f"l{layer}.mix.vmix"] = torch.tensor(val).to(torch.bfloat16)
+        d = tmp_path / sub
+        d.mkdir()
+        (d / "config.json").write_text(json.dumps(MIXED))
+        save_file({k: v.contiguous() for k, v in W2.items()}, str(d / "model.safetensors"))
+        return replay(engine(str(d), device), {"a": toks}, [[("a", 30)]])["a"], W2
+
+    first, _ = with_vmix(1, 0.9, "first")     # layer 1 is the first with value mixing
+    assert rel_err(first, base.double()) < 1e-6
+    later, W2 = with_vmix(3, 0.95, "later")
+    assert rel_err(later, base.double()) > 1e-2
+    assert rel_err(later, oracle.forward(MIXED, W2, toks)[0]) < 2e-4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("prefix_caching", [False, True], ids=["plain", "prefix-cache"])
+def test_greedy_generation_through_the_scheduler(tmp_path, device, prefix_caching):
+    path, W = model_dir(tmp_path, MIXED, seed=8)
+    shared = tokens(70, MIXED["vocab"], 21)
+    prompts = [tokens(9, MIXED["vocab"], 20), shared, tokens(1, MIXED["vocab"], 22), shared[:66] + [1, 2, 3]]
+    eng = engine(path, device, pages=10, seqs=2, async_scheduling=False,   # 4 requests over 2 places
+                 enable_prefix_caching=prefix_caching)
+    reqs = eng.generate(prompts, SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True))
+    for p, r in zip(prompts, reqs):
+        seq = list(p)
+        for _ in range(6):
+            seq.append(int(oracle.forward(MIXED, W, seq)[0][-1].argmax()))
+        assert r.output_token_ids == seq[len(p):]
+    eng.bm.check_invariants()
+
+
+def test_config_reads_every_size_from_the_file(tmp_path):
+    path, _ = model_dir(tmp_path, ODD)
+    mc = ModelConfig.from_hf(path)
+    assert mc.model_type == "negunex" and mc.hidden_size == 34 and mc.vocab_size == 51 and mc.hyper_streams == 4
+    assert mc.rms_norm_eps == 1e-4 and mc.num_hidden_layers == 3
+    assert [l["mixer"]["dim"] for l in mc.layer_specs] == [10, 18, 6]
+    assert ModelConfig.from_hf(PLAIN).hyper_streams == 0
+    bad = json.loads(json.dumps(ODD))
+    bad["layers"][1]["type"] = "something else"
+    with pytest.raises(ValueError):
+        ModelConfig.from_hf(bad)
+
+
+def test_trace_runner_program(tmp_path):
+    """bin/trace_run as a program on this design: a request that skips a step, ends, and a later one
+    that takes over its pages."""
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    path, W = model_dir(tmp_path, ONE_STREAM, seed=3)
+    V = ONE_STREAM["vocab"]
+    a, b, c = (tokens(n, V, 40 + i) for i, n in enumerate((70, 3, 5)))
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:62], "want": [0, 61]}, {"id": "b", "tokens": b[:2], "want": []}],
+              "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[62:63], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[2:], "want": [0]}, {"id": "a", "tokens": a[63:], "want": [1, 6]}],
+              "end": ["a", "b"]},
+             {"step": 3, "entries": [{"id": "c", "tokens": c, "want": [4]}], "end": ["c"]}]
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "192", "--max-seqs", "2", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    la, lb, lc = (oracle.forward(ONE_STREAM, W, t)[0] for t in (a, b, c))
+    want = {0: torch.stack([la[0], la[61]]), 1: la[62:63], 2: torch.stack([lb[2], la[64], la[69]]), 3: lc[4:5]}
+    for i, w in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V).copy())
+        assert got.shape == w.shape and rel_err(got, w) < 2e-4, i
