@@ -92,9 +92,13 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--mixer-bench", action="store_true",
                    help="instead of the serving workload: prefill / decode throughput of the per-layer stacks "
-                        "(latent attention + experts, selective scan, delta rule) at model-like sizes beside "
-                        "DeepSeek-V2-Lite layers of equal size (llmd_amd/tools/mixer_bench.py; uses --isl as "
+                        "(latent attention + experts, selective scan, delta rule beside DeepSeek-V2-Lite layers; "
+                        "hyper-connected grouped attention beside Llama-3-8B and Qwen3-30B-A3B layers) at model-like "
+                        "sizes (llmd_amd/tools/mixer_bench.py; uses --isl as "
                         "the context and --concurrency as the decode batch when they are given)")
+    p.add_argument("--mixer-only", default="",
+                   help="with --mixer-bench: only the entries whose name starts with one of these (commas between), "
+                        "e.g. negunex,llama,qwen3")
     p.add_argument("--steps", type=int, default=40)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--model", default="llama-3-70b")
@@ -158,7 +162,7 @@ def main():
         from llmd_amd.tools import mixer_bench
 
         ctx = a.isl if a.isl != 5000 else 2048
-        print(json.dumps(mixer_bench.run(tokens=ctx, batch=min(a.concurrency, 64))), flush=True)
+        print(json.dumps(mixer_bench.run(tokens=ctx, batch=min(a.concurrency, 64), only=a.mixer_only)), flush=True)
         return
     if os.environ.get("LLMD_BENCH_STACKS"):
         import faulthandler

@@ -38,7 +38,7 @@ void sm_qkv_rope_cache(const void*, int64_t, const float*, const int64_t*, const
 int sm_grouped_attention(const void*, const void*, const int*, int, int, const int*, const int*, float, int, int, int,
                          int, int, int, const void*, int64_t, void*, int, hipStream_t);
 int sm_grouped_attention_mfma(const void*, const void*, const int*, int, int, const int*, int, const int*, float, int,
-                              int, int, int, const void*, int64_t, void*, int, int, float*, float*, hipStream_t);
+                              int, int, int, const void*, int64_t, void*, int, int, float*, float*, int, hipStream_t);
 void sm_moe_route_scores(const float*, const float*, int, int, int*, float*, int, hipStream_t);
 void sm_moe_route(const float*, int, int, int*, float*, int, hipStream_t);
 void sm_moe_group(const int*, int, int, int*, int*, int*, int, hipStream_t);
@@ -436,7 +436,8 @@ void grouped_attention(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor
 
 bool grouped_attention_mfma(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor tables, Tensor items,
                             Tensor row_len, double scale, std::optional<Tensor> gate, Tensor out, int64_t nsplit,
-                            int64_t split_keys, std::optional<Tensor> part_o, std::optional<Tensor> part_ml) {
+                            int64_t split_keys, std::optional<Tensor> part_o, std::optional<Tensor> part_ml,
+                            int64_t rb) {
   const c10::hip::OptionalHIPGuard g(dev_of(q));
   check_gqa(q, cache, dim, vdim, tables, row_len, gate, out);
   TORCH_CHECK(q.scalar_type() == torch::kBFloat16, "bf16 only");
@@ -444,7 +445,7 @@ bool grouped_attention_mfma(Tensor q, Tensor cache, int64_t dim, int64_t vdim, T
   TORCH_CHECK(items.dim() == 2 && items.size(1) == 3, "items [n, 3]");
   const int64_t n = items.size(0), Hkv = cache.size(1);
   float *po = nullptr, *pm = nullptr;
-  TORCH_CHECK(nsplit >= 1, "nsplit");
+  TORCH_CHECK(nsplit >= 1 && (rb == 1 || rb == 2) && (nsplit == 1 || rb == 1), "nsplit / rows per wave");
   if (nsplit > 1) {
     TORCH_CHECK(part_o && part_ml && split_keys > 0 && split_keys % 32 == 0, "split workspace");
     CHECK_F32(*part_o);
@@ -458,7 +459,7 @@ bool grouped_attention_mfma(Tensor q, Tensor cache, int64_t dim, int64_t vdim, T
                                            cache.size(2), items.data_ptr<int>(), n, row_len.data_ptr<int>(),
                                            (float)scale, q.size(1), Hkv, dim, vdim, gate ? gate->data_ptr() : nullptr,
                                            gate ? gate->stride(0) : 0, out.data_ptr(), nsplit, split_keys, po, pm,
-                                           cur());
+                                           rb, cur());
   return rc == 0;
 }
 

@@ -1,5 +1,8 @@
-// Grouped-query softmax attention with separate key and value sizes over a paged cache whose
-// row per (token, kv head) is [key (dim) | value (vdim)]: cache [blocks, Hkv, bs, dim + vdim].
+// Grouped-query softmax attention with separate key and value sizes over a paged cache. A page of
+// one kv head holds bs * (dim + vdim) elements: the keys [bs, dim] row-major, then the values
+// TRANSPOSED [vdim, bs] - a value column's keys are contiguous, so both tiles of the matrix-core
+// kernel are 16-byte loads and 16-byte LDS writes with nothing to transpose. The cache tensor is
+// [blocks, Hkv, bs, dim + vdim] by size only.
 //
 // qkv_rope_cache: one workgroup per token over the fused projection [q | k | v | ...]: bias add,
 //   rotary on the first rot_dims dimensions of every q and k head (pairs (2i, 2i+1) or
@@ -9,11 +12,12 @@
 // grouped_attention (fp32 FMA form): workgroup = QT consecutive token rows x up to 4 query heads
 //   of ONE kv head (a wave per head). Keys and values stream through LDS in fp32 tiles; a lane
 //   scores one key, the wave keeps an online softmax per (row, head), lanes then own value columns.
-// grouped_attention_mfma (bf16): a workgroup takes one work item - up to 64 (token, head of the
-//   group) rows of one sequence and kv head, 16 rows per wave. Key tiles of 32 in LDS (keys
-//   row-major, values transposed), S^T = K Q^T and O += P V on v_mfma_f32_16x16x32_bf16; fp32
-//   online softmax; P enters the second product as a bf16 pair (hi + lo). Decode-only steps cut
-//   the keys into ranges over blockIdx.z and a merge kernel joins them.
+// grouped_attention_mfma (bf16): a workgroup takes one work item - up to 64 or 128 (token, head of
+//   the group) rows of one sequence and kv head, one or two blocks of 16 rows per wave. Key tiles of
+//   32 in LDS (keys row-major, values transposed as in the cache), S^T = K Q^T and O += P V on
+//   v_mfma_f32_16x16x32_bf16; fp32 online softmax in base 2; P enters the second product as a bf16
+//   pair (hi + lo). Decode-only steps cut the keys into ranges over blockIdx.z and a merge kernel
+//   joins them.
 // Both forms multiply the result by sigmoid(gate) when a gate is given. A row's result depends
 // only on its own keys and the fixed tile sizes.
 #include "seqmix_common.h"
@@ -75,7 +79,7 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
     if (unit) inv = 1.f / sqrtf(wave_sum(ss) / (float)dim + eps);
     T* dst = nullptr;
     if (is_q) dst = q_out + (t * Hq + hd) * dim;
-    else if (slot >= 0) dst = cache + ((blk * Hkv + (hd - Hq)) * bs + off) * Dr;
+    else if (slot >= 0) dst = cache + (blk * Hkv + (hd - Hq)) * bs * Dr + off * dim;
     if (dst == nullptr) continue;
 #pragma unroll
     for (int i = 0; i < MAXE; ++i) {
@@ -90,7 +94,7 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
     else if (v_mode == 2) v = (1.f - lam) * v + lam * v_first[t * nv + e];
     if (slot >= 0) {
       const int g = e / vdim, c = e - g * vdim;
-      st(cache + ((blk * Hkv + g) * bs + off) * Dr + dim + c, v);
+      st(cache + (blk * Hkv + g) * bs * Dr + (int64_t)bs * dim + (int64_t)c * bs + off, v);  // transposed
     }
   }
 }
@@ -155,15 +159,20 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
     const int* bt = tables + (int64_t)seq * W;
     for (int k0 = 0; k0 < maxlen; k0 += KT) {
       __syncthreads();  // previous tile fully used (and sQ written, first time)
-      for (int e = threadIdx.x; e < KT * Dr; e += NT) {
-        const int j = e / Dr, d = e - j * Dr;
+      for (int e = threadIdx.x; e < KT * dim; e += NT) {  // keys: row-major in the page
+        const int j = e / dim, d = e - j * dim;
         const int key = k0 + j;
         float v = 0.f;
-        if (key < maxlen) {
-          const int64_t rowi = ((int64_t)bt[key / bs] * Hkv + g) * bs + (key % bs);
-          v = ld(cache + rowi * Dr + d);
-        }
+        if (key < maxlen) v = ld(cache + ((int64_t)bt[key / bs] * Hkv + g) * bs * Dr + (int64_t)(key % bs) * dim + d);
         sK[j * KS + d] = v;
+      }
+      for (int e = threadIdx.x; e < KT * vdim; e += NT) {  // values: transposed in the page, lanes along keys
+        const int d = e / KT, j = e - d * KT;
+        const int key = k0 + j;
+        float v = 0.f;
+        if (key < maxlen)
+          v = ld(cache + ((int64_t)bt[key / bs] * Hkv + g) * bs * Dr + (int64_t)bs * dim + (int64_t)d * bs + (key % bs));
+        sK[j * KS + dim + d] = v;
       }
       __syncthreads();
       if (!head_ok) continue;
@@ -224,8 +233,11 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int MKT = 32;  // keys per tile
 
 // DkP = 32 NKS >= dim and VP = 16 NCB >= vdim are the padded sizes (zeros in LDS and in the
-// query fragments). items [n, 3] = (sequence, first token row, tokens), tokens * G <= 64.
-template <int NKS, int NCB>
+// query fragments). items [n, 3] = (sequence, first token row, tokens), tokens * G <= 64 RB: a wave
+// owns RB blocks of 16 rows (block rb of wave w = item rows 16 (4 rb + w) ..), so a key tile's
+// fragments are read from LDS once for RB row blocks. The next tile's global loads are issued
+// before the current tile's products, so their latency runs beside the matrix work.
+template <int NKS, int NCB, int RB>
 __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
     const int* __restrict__ items, const int* __restrict__ row_len, float scale, int Hq, int Hkv, int dim, int vdim,
@@ -235,161 +247,221 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   constexpr int KS = DkP + 8, VS = MKT + 8, PS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
   __shared__ __attribute__((aligned(16))) bf16_t sK[MKT * KS];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[VP * VS];
-  __shared__ __attribute__((aligned(16))) bf16_t sP[2 * 4 * 16 * PS];
-  bf16_t* const sPh = sP;
-  bf16_t* const sPl = sP + 4 * 16 * PS;
+  __shared__ __attribute__((aligned(16))) bf16_t sP[2 * RB * 4 * 16 * PS];  // [hi | lo][rb][wave][16][PS]
   const int seq = items[blockIdx.x * 3], tok0 = items[blockIdx.x * 3 + 1], ntok = items[blockIdx.x * 3 + 2];
   const int g = blockIdx.y, G = Hq / Hkv, Dr = dim + vdim;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, kq = lane >> 4;
-  // this lane's query row (as the B operand's column): item row 16 wave + r16
-  const int myrow = wave * 16 + r16;
-  const bool row_ok = myrow < ntok * G;
-  const int mytok = tok0 + (row_ok ? myrow / G : 0), myhead = g * G + (row_ok ? myrow % G : 0);
-  const int mylen = row_ok ? row_len[mytok] : 0;
+  // this lane's query rows (as the B operand's column): item row 16 (4 rb + wave) + r16
+  int mytok[RB], myhead[RB], mylen[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int myrow = (rb * 4 + wave) * 16 + r16;
+    const bool ok = myrow < ntok * G;
+    mytok[rb] = tok0 + (ok ? myrow / G : 0);
+    myhead[rb] = g * G + (ok ? myrow % G : 0);
+    mylen[rb] = ok ? row_len[mytok[rb]] : 0;
+  }
   const int maxlen = row_len[tok0 + ntok - 1];  // the run's last token sees the most keys
 
   // padding columns of the key tile and padding rows of the value tile stay zero for the whole kernel
   for (int e = threadIdx.x; e < MKT * KS; e += NT) sK[e] = 0;
   for (int e = threadIdx.x; e < VP * VS; e += NT) sVt[e] = 0;
 
-  bf16x8_t qf[NKS];
+  bf16x8_t qf[RB][NKS];
 #pragma unroll
-  for (int ks = 0; ks < NKS; ++ks) {
+  for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int d = ks * 32 + kq * 8 + i;
-      const bf16_t w = (row_ok && d < dim) ? q[((int64_t)mytok * Hq + myhead) * dim + d] : (bf16_t)0;
-      qf[ks][i] = __builtin_bit_cast(__bf16, w);
+    for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int d = ks * 32 + kq * 8 + i;
+        const bf16_t w = (mylen[rb] > 0 && d < dim) ? q[((int64_t)mytok[rb] * Hq + myhead[rb]) * dim + d] : (bf16_t)0;
+        qf[rb][ks][i] = __builtin_bit_cast(__bf16, w);
+      }
     }
-  }
-  f32x4_t o[NCB];
+  f32x4_t o[RB][NCB];
+  float m[RB], l[RB];
 #pragma unroll
-  for (int n = 0; n < NCB; ++n) o[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+  for (int rb = 0; rb < RB; ++rb) {
+    m[rb] = -INFINITY;
+    l[rb] = 0.f;
+#pragma unroll
+    for (int n = 0; n < NCB; ++n) o[rb][n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
   const int* bt = tables + (int64_t)seq * W;
-  bf16_t* ph = sPh + wave * 16 * PS;
-  bf16_t* pl = sPl + wave * 16 * PS;
-  const bool vec = (Dr & 7) == 0 && (dim & 7) == 0;
+  const bool vec = (dim & 7) == 0;  // key rows are 16-byte multiples (value columns always: bs % 8 == 0)
+  // the softmax runs in base 2 (scores carry log2 e): the hardware exponential is exp2, about one
+  // fp32 ulp, far below the bf16 rounding of what the weights multiply
+  const float scale2 = scale * 1.44269504088896341f;
 
   // decode steps split a row's keys over blockIdx.z: this workgroup takes [kbeg, kend)
   const int nsplit = gridDim.z;
   const int kbeg = nsplit > 1 ? blockIdx.z * split_keys : 0;
   const int kend = nsplit > 1 ? min(maxlen, kbeg + split_keys) : maxlen;
-  constexpr int CPR = (DkP + VP) / 8;             // 16-byte chunks per cache row (padded)
-  constexpr int NCH = (MKT * CPR + NT - 1) / NT;  // chunks per thread
-  const int cpr = (Dr + 7) / 8;                   // chunks that hold data
-  for (int k0 = kbeg; k0 < kend; k0 += MKT) {
-    __syncthreads();  // the previous tile is no longer read (first time: the zero fill is done)
-    // All of a tile's 16-byte chunks are requested before any is used. A tile lies inside one page
-    // when the page size is a multiple of the tile. Consecutive lanes take consecutive keys of one
-    // chunk, so the transposed 2-byte value writes fall into consecutive LDS words.
-    const bool one_page = (bs % MKT) == 0;
-    const int64_t row0 = one_page ? ((int64_t)bt[k0 / bs] * Hkv + g) * bs + (k0 % bs) : 0;
-    u32x4_t pre[NCH];
+  constexpr int CK = DkP / 8;                      // 16-byte chunks per key row (padded)
+  constexpr int NCK = (MKT * CK + NT - 1) / NT;    // key chunks per thread
+  constexpr int CV = MKT / 8;                      // chunks per value column (8 keys each)
+  constexpr int NCV = (VP * CV + NT - 1) / NT;     // value chunks per thread
+  const bool one_page = (bs % MKT) == 0;           // a tile lies inside one page (tiles start at multiples of 32)
+  // All of a tile's 16-byte chunks are requested before any is used: key rows with lanes along the
+  // row, value columns with lanes along the keys - both contiguous in the page. Keys at or beyond
+  // kend are zeroed (a page's unwritten rest may hold anything, and 0 x NaN would spoil a column).
+  u32x4_t pk[NCK], pv[NCV];
+  auto fetch = [&](int k0) {
+    const int64_t page0 = one_page ? ((int64_t)bt[k0 / bs] * Hkv + g) * bs * Dr : 0;
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
+    for (int i = 0; i < NCK; ++i) {
       const int e = threadIdx.x + i * NT;
-      const int c = e / MKT, j = e - c * MKT;
+      const int j = e / CK, c = e - j * CK;
       const int key = k0 + j;
       u32x4_t v = {0, 0, 0, 0};
-      if (c < cpr && key < kend) {
-        const int64_t row = one_page ? row0 + j : ((int64_t)bt[key / bs] * Hkv + g) * bs + (key % bs);
-        const bf16_t* src = cache + row * Dr + c * 8;
+      if (e < MKT * CK && c * 8 < dim && key < kend) {
+        const int64_t page = one_page ? page0 : ((int64_t)bt[key / bs] * Hkv + g) * bs * Dr;
+        const bf16_t* src = cache + page + (int64_t)(key % bs) * dim + c * 8;
         if (vec) {
           v = *reinterpret_cast<const u32x4_t*>(src);
         } else {
 #pragma unroll
           for (int qq = 0; qq < 8; ++qq)
-            if (c * 8 + qq < Dr) v[qq >> 1] |= (uint32_t)src[qq] << (16 * (qq & 1));
+            if (c * 8 + qq < dim) v[qq >> 1] |= (uint32_t)src[qq] << (16 * (qq & 1));
         }
       }
-      pre[i] = v;
+      pk[i] = v;
     }
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
+    for (int i = 0; i < NCV; ++i) {
       const int e = threadIdx.x + i * NT;
-      const int c = e / MKT, j = e - c * MKT;
-      if (c >= cpr) continue;
-      if (c * 8 + 8 <= dim) {
-        *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = pre[i];
-      } else {
+      const int d = e / CV, j8 = e - d * CV;
+      const int key = k0 + j8 * 8;
+      u32x4_t v = {0, 0, 0, 0};
+      if (d < vdim && key < kend) {
+        const int64_t page = one_page ? page0 : ((int64_t)bt[key / bs] * Hkv + g) * bs * Dr;
+        v = *reinterpret_cast<const u32x4_t*>(cache + page + (int64_t)bs * dim + (int64_t)d * bs + (key % bs));
+        const int nv = kend - key;  // keys of this chunk that exist
+        if (nv < 8) {
 #pragma unroll
-        for (int qq = 0; qq < 8; ++qq) {
-          const int d = c * 8 + qq;
-          const bf16_t val = (bf16_t)(pre[i][qq >> 1] >> (16 * (qq & 1)));
-          if (d < dim) sK[j * KS + d] = val;
-          else if (d < Dr) sVt[(d - dim) * VS + j] = val;
+          for (int w = 0; w < 4; ++w) v[w] = 2 * w + 1 < nv ? v[w] : (2 * w < nv ? v[w] & 0xffffu : 0u);
         }
       }
+      pv[i] = v;
+    }
+  };
+  if (kbeg < kend) fetch(kbeg);
+  for (int k0 = kbeg; k0 < kend; k0 += MKT) {
+    __syncthreads();  // the previous tile is no longer read (first time: the zero fill is done)
+#pragma unroll
+    for (int i = 0; i < NCK; ++i) {
+      const int e = threadIdx.x + i * NT;
+      const int j = e / CK, c = e - j * CK;
+      if (e < MKT * CK && c * 8 < dim) *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = pk[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NCV; ++i) {
+      const int e = threadIdx.x + i * NT;
+      const int d = e / CV, j8 = e - d * CV;
+      if (d < vdim) *reinterpret_cast<u32x4_t*>(&sVt[d * VS + j8 * 8]) = pv[i];
     }
     __syncthreads();
-    // scores of this lane's row against keys k0 + 16 kb + 4 kq + r
-    float sc[2][4];
+    if (k0 + MKT < kend) fetch(k0 + MKT);  // in flight during this tile's products
+    // scores of this lane's rows against keys k0 + 16 kb + 4 kq + r
+    float sc[RB][2][4];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
-      f32x4_t a = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      f32x4_t a[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) a[rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(&sK[(kb * 16 + r16) * KS + ks * 32 + kq * 8]);
-        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], a, 0, 0, 0);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) a[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[rb][ks], a[rb], 0, 0, 0);
       }
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        sc[kb][r] = (k0 + kb * 16 + kq * 4 + r < min(mylen, kend)) ? a[r] * scale : -INFINITY;
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          sc[rb][kb][r] = (k0 + kb * 16 + kq * 4 + r < min(mylen[rb], kend)) ? a[rb][r] * scale2 : -INFINITY;
     }
-    float mx = -INFINITY;
+    float cr[RB][4];
+    bool rescale[RB];  // wave-uniform: some row's maximum moved in this tile
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int rb = 0; rb < RB; ++rb) {
+      bf16_t* ph = sP + ((rb * 4 + wave) * 16) * PS;
+      bf16_t* pl = ph + RB * 4 * 16 * PS;
+      float mx = -INFINITY;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sc[kb][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float mn = fmaxf(m, mx);
-    const float mref = (mn == -INFINITY) ? 0.f : mn;  // a row with no key yet
-    const float corr = expf(m - mref);
-    float psum = 0.f;
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sc[rb][kb][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mn = fmaxf(m[rb], mx);
+      const float mref = (mn == -INFINITY) ? 0.f : mn;  // a row with no key yet
+      const float corr = __builtin_amdgcn_exp2f(m[rb] - mref);
+      float psum = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float pv = expf(sc[kb][r] - mref);
-        psum += pv;
-        const __bf16 hi = (__bf16)pv;
-        const __bf16 lo = (__bf16)(pv - (float)hi);
-        ph[r16 * PS + kb * 16 + kq * 4 + r] = __builtin_bit_cast(bf16_t, hi);
-        pl[r16 * PS + kb * 16 + kq * 4 + r] = __builtin_bit_cast(bf16_t, lo);
+      for (int kb = 0; kb < 2; ++kb) {
+        // this lane's four weights are four consecutive keys: one 8-byte LDS write each for hi and lo
+        uint32_t hw[2], lw[2];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float pv = __builtin_amdgcn_exp2f(sc[rb][kb][r] - mref);
+          psum += pv;
+          const __bf16 hi = (__bf16)pv;
+          const __bf16 lo = (__bf16)(pv - (float)hi);
+          const uint32_t hb = __builtin_bit_cast(bf16_t, hi), lb = __builtin_bit_cast(bf16_t, lo);
+          if (r & 1) {
+            hw[r >> 1] |= hb << 16;
+            lw[r >> 1] |= lb << 16;
+          } else {
+            hw[r >> 1] = hb;
+            lw[r >> 1] = lb;
+          }
+        }
+        *reinterpret_cast<uint2*>(&ph[r16 * PS + kb * 16 + kq * 4]) = make_uint2(hw[0], hw[1]);
+        *reinterpret_cast<uint2*>(&pl[r16 * PS + kb * 16 + kq * 4]) = make_uint2(lw[0], lw[1]);
       }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
-    l = l * corr + psum;
-    m = mn;
-    // the accumulators hold rows 4 kq + r: their correction comes from the lane that owns the row
-    float cr[4];
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      l[rb] = l[rb] * corr + psum;
+      m[rb] = mn;
+      // the accumulators hold rows 4 kq + r: their correction comes from the lane that owns the row
 #pragma unroll
-    for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, kq * 4 + r, 64);
-    // P is written and read by the same wave only: its own LDS writes are visible after a wave barrier
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      for (int r = 0; r < 4; ++r) cr[rb][r] = __shfl(corr, kq * 4 + r, 64);
+      rescale[rb] = __any(corr != 1.f);
+    }
+    // P is written and read by the same wave only: LDS operations of a wave complete in order
     __builtin_amdgcn_wave_barrier();
-    const bf16x8_t pah = *reinterpret_cast<const bf16x8_t*>(&ph[r16 * PS + kq * 8]);
-    const bf16x8_t pal = *reinterpret_cast<const bf16x8_t*>(&pl[r16 * PS + kq * 8]);
+    bf16x8_t pah[RB], pal[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const bf16_t* ph = sP + ((rb * 4 + wave) * 16) * PS;
+      pah[rb] = *reinterpret_cast<const bf16x8_t*>(&ph[r16 * PS + kq * 8]);
+      pal[rb] = *reinterpret_cast<const bf16x8_t*>(&ph[RB * 4 * 16 * PS + r16 * PS + kq * 8]);
+    }
 #pragma unroll
     for (int n = 0; n < NCB; ++n) {
       const bf16x8_t vb = *reinterpret_cast<const bf16x8_t*>(&sVt[(n * 16 + r16) * VS + kq * 8]);
-      f32x4_t acc = o[n];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[r] *= cr[r];
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pah, vb, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pal, vb, acc, 0, 0, 0);
-      o[n] = acc;
+      for (int rb = 0; rb < RB; ++rb) {
+        f32x4_t acc = o[rb][n];
+        if (rescale[rb]) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[r] *= cr[rb][r];
+        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pah[rb], vb, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pal[rb], vb, acc, 0, 0, 0);
+        o[rb][n] = acc;
+      }
     }
   }
-  // o[n][r] = O[row 4 kq + r][column 16 n + r16]
-  if (nsplit > 1) {
+  // o[rb][n][r] = O[row 16 (4 rb + wave) + 4 kq + r][column 16 n + r16]
+  if (nsplit > 1) {  // RB == 1 (the host splits decode-only steps, whose items have at most 64 rows)
     const int64_t pbase = (((int64_t)blockIdx.x * Hkv + g) * nsplit + blockIdx.z) * 64;
     if (kq == 0) {
-      part_ml[(pbase + myrow) * 2] = m;
-      part_ml[(pbase + myrow) * 2 + 1] = l;
+      part_ml[(pbase + wave * 16 + r16) * 2] = m[0];
+      part_ml[(pbase + wave * 16 + r16) * 2 + 1] = l[0];
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -397,32 +469,35 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
 #pragma unroll
       for (int n = 0; n < NCB; ++n) {
         const int col = n * 16 + r16;
-        if (col < vdim) part_o[(pbase + row) * vdim + col] = o[n][r];
+        if (col < vdim) part_o[(pbase + row) * vdim + col] = o[0][n][r];
       }
     }
     return;
   }
-  float inv[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) inv[r] = 1.f / __shfl(l, kq * 4 + r, 64);
+  for (int rb = 0; rb < RB; ++rb) {
+    float inv[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int row = wave * 16 + kq * 4 + r;
-    if (row >= ntok * G) continue;
-    const int64_t tok = tok0 + row / G;
-    const int h = g * G + row % G;
+    for (int r = 0; r < 4; ++r) inv[r] = 1.f / __shfl(l[rb], kq * 4 + r, 64);
 #pragma unroll
-    for (int n = 0; n < NCB; ++n) {
-      const int col = n * 16 + r16;
-      if (col >= vdim) continue;
-      float v = o[n][r] * inv[r];
-      if (gate) v *= 1.f / (1.f + expf(-ld(gate + tok * gate_stride + h * vdim + col)));
-      st(out + (tok * Hq + h) * vdim + col, v);
+    for (int r = 0; r < 4; ++r) {
+      const int row = (rb * 4 + wave) * 16 + kq * 4 + r;
+      if (row >= ntok * G) continue;
+      const int64_t tok = tok0 + row / G;
+      const int h = g * G + row % G;
+#pragma unroll
+      for (int n = 0; n < NCB; ++n) {
+        const int col = n * 16 + r16;
+        if (col >= vdim) continue;
+        float v = o[rb][n][r] * inv[r];
+        if (gate) v *= 1.f / (1.f + expf(-ld(gate + tok * gate_stride + h * vdim + col)));
+        st(out + (tok * Hq + h) * vdim + col, v);
+      }
     }
   }
 }
 
-// Merge the key-range partials of a split step: out = sum_z e^(m_z - M) o_z / sum_z e^(m_z - M) l_z.
+// Merge the key-range partials of a split step: out = sum_z 2^(m_z - M) o_z / sum_z 2^(m_z - M) l_z.
 __global__ __launch_bounds__(NT) void grouped_attention_merge_kernel(
     const int* __restrict__ items, int nsplit, const float* __restrict__ part_o, const float* __restrict__ part_ml,
     int Hq, int Hkv, int vdim, const bf16_t* __restrict__ gate, int64_t gate_stride, bf16_t* __restrict__ out) {
@@ -436,7 +511,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_merge_kernel(
   float L = 0.f;
   for (int z = 0; z < nsplit; ++z) {
     const float* ml = part_ml + ((base + z) * 64 + row) * 2;
-    L += expf(ml[0] - M) * ml[1];  // an empty range has m = -inf, l = 0
+    L += exp2f(ml[0] - M) * ml[1];  // maxima are in base 2; an empty range has m = -inf, l = 0
   }
   const int64_t tok = tok0 + row / G;
   const int h = g * G + row % G;
@@ -444,7 +519,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_merge_kernel(
     float a = 0.f;
     for (int z = 0; z < nsplit; ++z) {
       const int64_t pb = (base + z) * 64 + row;
-      a += expf(part_ml[pb * 2] - M) * part_o[pb * vdim + c];
+      a += exp2f(part_ml[pb * 2] - M) * part_o[pb * vdim + c];
     }
     float v = a / L;
     if (gate) v *= 1.f / (1.f + expf(-ld(gate + tok * gate_stride + h * vdim + c)));
@@ -518,23 +593,28 @@ int sm_grouped_attention(const void* q, const void* cache, const int* tables, in
   return 1;
 }
 
-// bf16, matrix cores. Returns 0, or 1 when the sizes are outside the compiled forms
+// bf16, matrix cores. ``rb`` (1 or 2): blocks of 16 rows per wave - items hold up to 64 rb rows;
+// key ranges (nsplit > 1) need rb = 1. Returns 0, or 1 when the sizes are outside the compiled forms
 // (dim > 256, vdim > 256, group size > 64).
 int sm_grouped_attention_mfma(const void* q, const void* cache, const int* tables, int W, int bs, const int* items,
                               int n_items, const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim,
                               const void* gate, int64_t gate_stride, void* out, int nsplit, int split_keys,
-                              float* part_o, float* part_ml, hipStream_t stream) {
+                              float* part_o, float* part_ml, int rb, hipStream_t stream) {
   if (n_items == 0) return 0;
   const int nks = (dim + 31) / 32, ncb = (vdim + 15) / 16;
-  if (Hq / Hkv > 64 || nks > 8 || ncb > 16) return 1;
+  if (Hq / Hkv > 64 || nks > 8 || ncb > 16 || (rb != 1 && rb != 2) || (nsplit > 1 && rb != 1) || bs % 8) return 1;
   const dim3 grid(n_items, Hkv, nsplit);
-#define SM_GO(NKS, NCB)                                                                                           \
-  hipLaunchKernelGGL((grouped_attention_mfma_kernel<NKS, NCB>), grid, dim3(NT), 0, stream, (const bf16_t*)q,       \
+#define SM_GO(NKS, NCB, RB)                                                                                       \
+  hipLaunchKernelGGL((grouped_attention_mfma_kernel<NKS, NCB, RB>), grid, dim3(NT), 0, stream, (const bf16_t*)q,   \
                      (const bf16_t*)cache, tables, W, bs, items, row_len, scale, Hq, Hkv, dim, vdim,               \
                      (const bf16_t*)gate, gate_stride, (bf16_t*)out, split_keys, part_o, part_ml)
-  if (nks <= 2 && ncb <= 4) SM_GO(2, 4);
-  else if (nks <= 4 && ncb <= 8) SM_GO(4, 8);
-  else SM_GO(8, 16);
+#define SM_GO2(NKS, NCB) \
+  if (rb == 2) SM_GO(NKS, NCB, 2); \
+  else SM_GO(NKS, NCB, 1)
+  if (nks <= 2 && ncb <= 4) { SM_GO2(2, 4); }
+  else if (nks <= 4 && ncb <= 8) { SM_GO2(4, 8); }
+  else { SM_GO2(8, 16); }
+#undef SM_GO2
 #undef SM_GO
   if (nsplit > 1)
     hipLaunchKernelGGL(grouped_attention_merge_kernel, dim3(n_items, Hkv, 64), dim3(NT), 0, stream, items, nsplit,

@@ -252,6 +252,7 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
 
 
 GQA_MFMA = os.environ.get("LLMD_GQA_MFMA", "1") == "1"
+GQA_RB_MIN = int(os.environ.get("LLMD_GQA_RB_MIN", "1"))  # runs longer than this many 64-row items take 128-row items
 
 
 def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
@@ -260,7 +261,7 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
     sequence. ``gate`` [T, Hq * vdim] (a column view of the fused projection): the result is
     multiplied by sigmoid(gate). Returns [T, Hq * vdim].
 
-    bfloat16 runs on the matrix cores (work item = up to 64 (token, head-of-group) rows of one
+    bfloat16 runs on the matrix cores (work item = up to 128 (token, head-of-group) rows of one
     sequence and kv head); float32 and sizes outside the compiled forms on the fp32 FMA kernel."""
     T, Hq, _ = q.shape
     Hkv = cache.shape[1]
@@ -269,19 +270,23 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
         return ref.grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, scale, gate, out)
     G = Hq // Hkv
     if GQA_MFMA and q.dtype == torch.bfloat16 and G <= 64:
-        items = seq.attention_items(max(1, 64 // G))
+        # prompt portions: two blocks of 16 rows per wave (items of up to 128 rows) once a run is
+        # long enough to fill them; single tokens: one block, and the keys cut into ranges
+        rb = 2 if seq.max_q * G > 64 * GQA_RB_MIN else 1
+        items = seq.attention_items(max(1, 64 * rb // G))
         nsplit, split, po, pm = 1, 0, None, None
         if seq.max_q == 1 and seq.max_len > 256:
-            # decode-only step: cut the keys into ranges so that items x kv heads x ranges fill the chip
+            # decode-only step: key ranges so that items x kv heads x ranges give the chip about
+            # eight workgroups per CU (a workgroup walks its tiles one after another)
             n = items.shape[0] * Hkv
-            nsplit = max(1, min(-(-512 // n), seq.max_len // 128))
+            nsplit = max(1, min(-(-2048 // n), seq.max_len // 128))
             split = -(-seq.max_len // (nsplit * 32)) * 32
             nsplit = -(-seq.max_len // split)
             if nsplit > 1:
                 po = torch.empty(n * nsplit * 64 * vdim, dtype=torch.float32, device=q.device)
                 pm = torch.empty(n * nsplit * 128, dtype=torch.float32, device=q.device)
         if native().grouped_attention_mfma(q, cache, dim, vdim, seq.tables, items, seq.row_len, float(scale), gate,
-                                           out, nsplit, split, po, pm):
+                                           out, nsplit, split, po, pm, rb):
             return out
     native().grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, float(scale), gate,
                                4 if seq.max_q > 1 else 1, out)

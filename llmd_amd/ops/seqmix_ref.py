@@ -201,23 +201,34 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
     elif v_mode == 2:
         v = (1.0 - lam) * v + lam * v_first.view(T, Hkv, vdim)
     q_out.copy_(q.to(q_out.dtype))
-    row = torch.cat([k, v], -1).to(cache.dtype)              # [T, Hkv, dim + vdim]
     nb, _, bs, _ = cache.shape
+    kc, vc = kv_views(cache, dim, vdim)
     ok = slots >= 0
     sl = slots[ok]
-    cache[sl // bs, :, sl % bs] = row[ok]
+    kc[sl // bs, :, sl % bs] = k[ok].to(cache.dtype)
+    vc[sl // bs, :, :, sl % bs] = v[ok].to(cache.dtype)
+
+
+def kv_views(cache, dim, vdim):
+    """The two parts of a page [Hkv, bs * (dim + vdim)] of the grouped-attention cache: keys
+    [blocks, Hkv, bs, dim] row-major, then values transposed [blocks, Hkv, vdim, bs] (a value
+    column's keys are contiguous, which is how the matrix cores read them)."""
+    nb, Hkv, bs, Dr = cache.shape
+    flat = cache.view(nb, Hkv, bs * Dr)
+    return flat[:, :, :bs * dim].view(nb, Hkv, bs, dim), flat[:, :, bs * dim:].view(nb, Hkv, vdim, bs)
 
 
 def grouped_attention(q, cache, dim, vdim, tables, row_seq, row_len, scale, gate, out):
     T, Hq, _ = q.shape
     nb, Hkv, bs, _ = cache.shape
     G = Hq // Hkv
+    kc, vc = kv_views(cache, dim, vdim)
     for t in range(T):
         n = int(row_len[t])
         bt = tables[int(row_seq[t])].long()
         ar = torch.arange(n)
-        rows = cache[bt[ar // bs], :, ar % bs].float()        # [n, Hkv, dim + vdim]
-        K, V = rows[..., :dim], rows[..., dim:]
+        K = kc[bt[ar // bs], :, ar % bs].float()              # [n, Hkv, dim]
+        V = vc[bt[ar // bs], :, :, ar % bs].float()           # [n, Hkv, vdim]
         qt = q[t].float().view(Hkv, G, dim)
         s = torch.einsum("hgd,nhd->hgn", qt, K) * scale
         o = torch.einsum("hgn,nhv->hgv", torch.softmax(s, -1), V).reshape(Hq * vdim)

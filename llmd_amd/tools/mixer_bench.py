@@ -11,6 +11,14 @@ Mekusun stacks of DeepSeek-V2-Lite's width (2048) are timed through the runner's
   mamba      : selective scan, inner 4096, state 16, dt rank 128, 4 taps; dense ff 5632
   delta      : generalized delta rule, 32 heads x 64; dense ff 5632
 
+Two Negunex stacks (grouped attention with value mixing and an output gate over two
+hyper-connected streams) run beside the existing models of the same layer geometry:
+
+  negunex-dense : width 4096, 32 heads / 8 kv heads x 128, value 128, dense ff 14336 - beside
+                  Llama-3-8B layers (models/llama.py)
+  negunex-moe   : width 2048, 32 heads / 4 kv heads x 128, 128 experts + 4 identity, 8 chosen, ff 768 -
+                  beside Qwen3-30B-A3B layers (models/moe_llama.py)
+
 Prefill: one prompt of ``--tokens`` tokens in one step. Decode: ``--batch`` sequences with that
 context, one token each. One JSON line with tokens/s and ms per layer for every entry.
 """
@@ -51,6 +59,18 @@ def stack_config(layer: dict, n_layers: int):
                            "logit_softcap": 30.0, "norm": {"eps": 1e-6}, "layers": [layer] * n_layers})
 
 
+def _negunex(width, heads, kv, ff=None, experts=None):
+    from llmd_amd.engine.config import negunex_config
+
+    rot = {"dims": 128, "base": 500000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    mixer = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "v_mix": True, "rot": rot}
+    mlp = {"kind": "dense", "ff": ff} if ff else \
+        {"kind": "moe", "expert": {"ff": experts[2]}, "router": {"experts": experts[0], "identity": 4, "top": experts[1]}}
+    return lambda n: negunex_config({"architecture": "Negunex", "width": width, "vocab": 32000, "streams": 2,
+                                     "norm": {"eps": 1e-6},
+                                     "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp}] * n})
+
+
 def _runner(mc, tokens: int, batch: int, device: str):
     from llmd_amd.engine.config import EngineConfig
     from llmd_amd.engine.model_runner import ModelRunner
@@ -81,9 +101,9 @@ def _plans(r, tokens: int, batch: int):
            "slots": [int(d_bt[b, tokens // bs]) * bs + tokens % bs for b in range(batch)], "d_bt": d_bt,
            "d_len": np.full(batch, tokens + 1, np.int32), "p_ql": [], "p_ctx": [],
            "p_bt": np.zeros((0, W), np.int32), "rows": list(range(batch))}
-    if r.stateful:
+    if r.seq_steps:
         pre["seq"] = ([0], [0])
-        dec["seq"] = (list(range(1, batch + 1)), [1] * batch)
+        dec["seq"] = (list(range(1, batch + 1)) if r.stateful else [0] * batch, [1] * batch)
     return pre, dec
 
 
@@ -108,9 +128,15 @@ def run(tokens: int = 2048, batch: int = 32, n_layers: int = 4, reps: int = 5, d
     ref = dataclasses.replace(get_model_config("deepseek-v2-lite"), num_hidden_layers=n_layers + 1,
                               first_k_dense_replace=1, vocab_size=32000, rope_scaling=None, name="deepseek-v2-lite-cut")
     todo = [("latent+moe", stack_config(_attn(), n_layers), n_layers), ("mamba", stack_config(_mamba(), n_layers), n_layers),
-            ("delta", stack_config(_delta(), n_layers), n_layers), ("deepseek-v2-lite (1 dense + moe layers)", ref, n_layers + 1)]
+            ("delta", stack_config(_delta(), n_layers), n_layers), ("deepseek-v2-lite (1 dense + moe layers)", ref, n_layers + 1),
+            ("negunex-dense", _negunex(4096, 32, 8, ff=14336)(n_layers), n_layers),
+            ("llama-3-8b layers", dataclasses.replace(get_model_config("llama-3-8b"), num_hidden_layers=n_layers,
+                                                      vocab_size=32000, name="llama-3-8b-cut"), n_layers),
+            ("negunex-moe", _negunex(2048, 32, 4, experts=(128, 8, 768))(n_layers), n_layers),
+            ("qwen3-30b-a3b layers", dataclasses.replace(get_model_config("qwen3-30b-a3b"), num_hidden_layers=n_layers,
+                                                         vocab_size=32000, name="qwen3-30b-a3b-cut"), n_layers)]
     for name, mc, L in todo:
-        if only and not name.startswith(only):
+        if only and not any(name.startswith(o) for o in only.split(",")):
             continue
         r = _runner(mc, tokens, batch, device)
         pre, dec = _plans(r, tokens, batch)
@@ -128,7 +154,7 @@ def main(argv=None):
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--layers", type=int, default=4)
     ap.add_argument("--reps", type=int, default=5)
-    ap.add_argument("--only", default="", help="run the entries whose name starts with this")
+    ap.add_argument("--only", default="", help="run the entries whose name starts with one of these (commas between)")
     a = ap.parse_args(argv)
     print(json.dumps(run(a.tokens, a.batch, a.layers, a.reps, only=a.only)), flush=True)
 

@@ -136,6 +136,24 @@ def _dev(t, device, dtype=None):
     return (t if dtype is None else t.to(dtype)).to(device)
 
 
+def _rows_of(cache, dim):
+    """The cache's pages as rows: [blocks, Hkv, bs, dim + vdim] with row = [key | value]. A page of one kv
+    head stores its keys [bs, dim] first and then its values transposed [vdim, bs]."""
+    nb, Hkv, bs, Dr = cache.shape
+    flat = cache.reshape(nb, Hkv, bs * Dr)
+    k = flat[:, :, :bs * dim].reshape(nb, Hkv, bs, dim)
+    v = flat[:, :, bs * dim:].reshape(nb, Hkv, Dr - dim, bs).transpose(2, 3)
+    return torch.cat([k, v], -1)
+
+
+def _pages_of(rows, dim):
+    """Inverse of _rows_of."""
+    nb, Hkv, bs, Dr = rows.shape
+    k = rows[..., :dim].reshape(nb, Hkv, bs * dim)
+    v = rows[..., dim:].transpose(2, 3).reshape(nb, Hkv, (Dr - dim) * bs)
+    return torch.cat([k, v], -1).reshape(nb, Hkv, bs, Dr).contiguous()
+
+
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("S,d", [(1, 40), (2, 33), (5, 300)])
 def test_streams_and_layer_norm(device, S, d):
@@ -221,7 +239,7 @@ def test_projection_rotary_norm_cache(device, interleaved, Hq, Hkv, dim, vdim, r
         if mode == 2:
             v = (1 - lam) * v + lam * vf.double().view(T, Hkv, vdim)
         assert rel_err(q_d, q) < 1e-5
-        got = cache_d.cpu()
+        got = _rows_of(cache_d.cpu(), dim)
         for t in range(T):
             s = int(slots[t])
             if s < 0:
@@ -234,7 +252,7 @@ def test_projection_rotary_norm_cache(device, interleaved, Hq, Hkv, dim, vdim, r
         assert float(got.permute(0, 2, 1, 3).reshape(3 * bs, -1)[mask].abs().max()) == 0.0  # nothing else is touched
 
 
-def _paged(rows, bs, device, dtype, seed=1):
+def _paged(rows, bs, device, dtype, dim, seed=1):
     """rows [n, Hkv, Dr] scattered over shuffled pages of a cache filled with noise; (cache, table row)."""
     n, Hkv, Dr = rows.shape
     nb = -(-n // bs)
@@ -242,7 +260,7 @@ def _paged(rows, bs, device, dtype, seed=1):
     cache = torch.randn(nb + 3, Hkv, bs, Dr, generator=torch.Generator().manual_seed(seed + 1)).to(dtype)
     for i in range(n):
         cache[perm[i // bs], :, i % bs] = rows[i].to(dtype)
-    return cache.to(device), perm.int()
+    return _pages_of(cache, dim).to(device), perm.int()
 
 
 def _seq_meta(device, tables, q_lens, lens):
@@ -299,7 +317,7 @@ def test_one_key_stands_out(device, dtype, where, decode):
     rows[j, 1, :dim] = q[-1, h] / q[-1, h].norm() * 12.0   # and looks straight at key j
     q[-1, h] *= 6.0
     rows, q = rows.to(dtype).float(), q.to(dtype).float()  # the values both sides compute with
-    cache, table = _paged(rows, 64, device, dtype)
+    cache, table = _paged(rows, 64, device, dtype, dim)
     seq = _seq_meta(device, [table], [nq], [seen])
     gate = torch.randn(nq, Hq * vdim, generator=g).to(dtype)
     out = sm.grouped_attention(q.to(dtype).to(device), cache, dim, vdim, 1.0, seq, gate.to(device))
@@ -338,7 +356,7 @@ def test_grouped_attention_steps(device, dtype, Hq, Hkv, dim, vdim, decode_only)
     T = sum(q_lens)
     q = (torch.randn(T, Hq, dim, generator=g) * 0.5).to(dtype)
     gate = torch.randn(T, Hq * vdim + 8, generator=g).to(dtype)[:, 3:3 + Hq * vdim]  # a strided column view
-    out = sm.grouped_attention(q.to(device), cache.to(device), dim, vdim, 0.3, seq, gate.to(device))
+    out = sm.grouped_attention(q.to(device), _pages_of(cache, dim).to(device), dim, vdim, 0.3, seq, gate.to(device))
     t0 = 0
     for rows, c, n in zip(all_rows, q_lens, lens):
         want = _attention_oracle(q[t0:t0 + c].float(), rows, dim, [n - c + i + 1 for i in range(c)], 0.3,
