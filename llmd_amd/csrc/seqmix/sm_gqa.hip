@@ -248,8 +248,9 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t sK[MKT * KS];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[VP * VS];
   __shared__ __attribute__((aligned(16))) bf16_t sP[2 * RB * 4 * 16 * PS];  // [hi | lo][rb][wave][16][PS]
-  const int seq = items[blockIdx.x * 3], tok0 = items[blockIdx.x * 3 + 1], ntok = items[blockIdx.x * 3 + 2];
-  const int g = blockIdx.y, G = Hq / Hkv, Dr = dim + vdim;
+  // the kv head is the fastest grid index: the workgroups of one item follow each other
+  const int item = blockIdx.y, g = blockIdx.x, G = Hq / Hkv, Dr = dim + vdim;
+  const int seq = items[item * 3], tok0 = items[item * 3 + 1], ntok = items[item * 3 + 2];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, kq = lane >> 4;
   // this lane's query rows (as the B operand's column): item row 16 (4 rb + wave) + r16
@@ -458,7 +459,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   }
   // o[rb][n][r] = O[row 16 (4 rb + wave) + 4 kq + r][column 16 n + r16]
   if (nsplit > 1) {  // RB == 1 (the host splits decode-only steps, whose items have at most 64 rows)
-    const int64_t pbase = (((int64_t)blockIdx.x * Hkv + g) * nsplit + blockIdx.z) * 64;
+    const int64_t pbase = (((int64_t)item * Hkv + g) * nsplit + blockIdx.z) * 64;
     if (kq == 0) {
       part_ml[(pbase + wave * 16 + r16) * 2] = m[0];
       part_ml[(pbase + wave * 16 + r16) * 2 + 1] = l[0];
@@ -603,7 +604,8 @@ int sm_grouped_attention_mfma(const void* q, const void* cache, const int* table
   if (n_items == 0) return 0;
   const int nks = (dim + 31) / 32, ncb = (vdim + 15) / 16;
   if (Hq / Hkv > 64 || nks > 8 || ncb > 16 || (rb != 1 && rb != 2) || (nsplit > 1 && rb != 1) || bs % 8) return 1;
-  const dim3 grid(n_items, Hkv, nsplit);
+  if (n_items > 65535) return 1;
+  const dim3 grid(Hkv, n_items, nsplit);
 #define SM_GO(NKS, NCB, RB)                                                                                       \
   hipLaunchKernelGGL((grouped_attention_mfma_kernel<NKS, NCB, RB>), grid, dim3(NT), 0, stream, (const bf16_t*)q,   \
                      (const bf16_t*)cache, tables, W, bs, items, row_len, scale, Hq, Hkv, dim, vdim,               \

@@ -28,24 +28,42 @@ class SeqMeta:
     max_len: int = 0                 # longest context of the step
     max_q: int = 0                   # longest run of the step
     q_lens: Optional[list] = None    # host copy of the run lengths
-    _items: Optional[dict] = None    # tokens per item -> [n, 3] int32 work items (attention_items)
+    ctx_lens: Optional[list] = None  # host copy of each sequence's context length after the step
+    _items: Optional[dict] = None    # (tokens per item, balance) -> [n, 3] int32 work items (attention_items)
 
-    def attention_items(self, tokens_per_item: int) -> torch.Tensor:
+    def attention_items(self, tokens_per_item: int, balance: int = 0) -> torch.Tensor:
         """Work items (sequence, first token row, tokens) of the matrix-core attention kernel: every
-        run cut into pieces of at most ``tokens_per_item`` tokens. Built once per step and size."""
+        run cut into pieces of at most ``tokens_per_item`` tokens. Built once per step and size.
+
+        ``balance`` > 0 (needs ``ctx_lens``): a causal item's work grows with its position in the
+        prompt, and the workgroups of a step are all resident at once, dealt to the CUs in order. The
+        items are sorted by their number of keys and laid out as a snake over blocks of ``balance``
+        items (descending, ascending, descending, ...), so that the workgroups that land on one CU -
+        one of every block - sum to about the same number of key tiles."""
         if self._items is None:
             self._items = {}
-        it = self._items.get(tokens_per_item)
+        key = (tokens_per_item, balance if self.ctx_lens is not None else 0)
+        it = self._items.get(key)
         if it is None:
-            rows, t0 = [], 0
+            rows, keys, t0 = [], [], 0
             for s, n in enumerate(self.q_lens):
                 for a in range(0, n, tokens_per_item):
-                    rows.append((s, t0 + a, min(tokens_per_item, n - a)))
+                    c = min(tokens_per_item, n - a)
+                    rows.append((s, t0 + a, c))
+                    if key[1]:
+                        keys.append(self.ctx_lens[s] - n + a + c)
                 t0 += n
+            if key[1] and len(rows) > 1:
+                order = sorted(range(len(rows)), key=lambda i: -keys[i])
+                snake = []
+                for b in range(0, len(order), balance):
+                    blk = order[b:b + balance]
+                    snake.extend(blk if (b // balance) % 2 == 0 else blk[::-1])
+                rows = [rows[i] for i in snake]
             it = torch.tensor(rows, dtype=torch.int32).view(-1, 3)
             if self.tables.is_cuda:
                 it = it.pin_memory().to(self.tables.device, non_blocking=True)
-            self._items[tokens_per_item] = it
+            self._items[key] = it
         return it
 
 

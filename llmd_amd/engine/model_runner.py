@@ -833,7 +833,7 @@ class ModelRunner:
                        row_seq=sd[o[3]:o[4]], row_len=sd[o[4]:o[5]],
                        tables=torch.from_numpy(np.ascontiguousarray(tables)).to(dev, non_blocking=True),
                        max_len=int(row_len.max()) if T else 0, max_q=int(ql.max()) if n else 0,
-                       q_lens=ql.tolist())
+                       q_lens=ql.tolist(), ctx_lens=[int(x) for x in pl["d_len"]] + [int(x) for x in p_ctx])
 
     @torch.no_grad()
     def forward_logits(self, so: SchedulerOutput, block_tables: dict, rows: list[int]):

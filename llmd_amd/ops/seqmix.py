@@ -252,7 +252,10 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
 
 
 GQA_MFMA = os.environ.get("LLMD_GQA_MFMA", "1") == "1"
-GQA_RB_MIN = int(os.environ.get("LLMD_GQA_RB_MIN", "1"))  # runs longer than this many 64-row items take 128-row items
+# LLMD_GQA_RB2=1: prompt portions run as 128-row items, two blocks of 16 rows per wave. Measured slower
+# than 64-row items at 128/128 heads (2048-token prompt: 227 us against 181 us - 185 + 64 registers
+# leave two waves per SIMD instead of three), so it stays an option.
+GQA_RB2 = os.environ.get("LLMD_GQA_RB2", "0") == "1"
 
 
 def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
@@ -261,7 +264,7 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
     sequence. ``gate`` [T, Hq * vdim] (a column view of the fused projection): the result is
     multiplied by sigmoid(gate). Returns [T, Hq * vdim].
 
-    bfloat16 runs on the matrix cores (work item = up to 128 (token, head-of-group) rows of one
+    bfloat16 runs on the matrix cores (work item = up to 64 (token, head-of-group) rows of one
     sequence and kv head); float32 and sizes outside the compiled forms on the fp32 FMA kernel."""
     T, Hq, _ = q.shape
     Hkv = cache.shape[1]
@@ -270,10 +273,9 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
         return ref.grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, scale, gate, out)
     G = Hq // Hkv
     if GQA_MFMA and q.dtype == torch.bfloat16 and G <= 64:
-        # prompt portions: two blocks of 16 rows per wave (items of up to 128 rows) once a run is
-        # long enough to fill them; single tokens: one block, and the keys cut into ranges
-        rb = 2 if seq.max_q * G > 64 * GQA_RB_MIN else 1
-        items = seq.attention_items(max(1, 64 * rb // G))
+        rb = 2 if GQA_RB2 and seq.max_q * G > 64 else 1
+        # workgroup ids run over the kv heads first: ids 256 apart (256 // Hkv items apart) share a CU
+        items = seq.attention_items(max(1, 64 * rb // G), balance=max(1, 256 // Hkv) if seq.max_q > 1 else 0)
         nsplit, split, po, pm = 1, 0, None, None
         if seq.max_q == 1 and seq.max_len > 256:
             # decode-only step: key ranges so that items x kv heads x ranges give the chip about
