@@ -478,6 +478,31 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ 
   }
 }
 
+// bf16 rows that are 16-byte multiples: a thread sums eight columns from 16-byte loads.
+__global__ __launch_bounds__(256) void moe_combine_vec_kernel(const bf16_t* __restrict__ y,
+                                                              const int* __restrict__ pair_slot,
+                                                              const float* __restrict__ w, int k, int d,
+                                                              bf16_t* __restrict__ out, const bf16_t* __restrict__ h) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x * 8; c < d; c += 256 * 8) {
+    float s[8] = {};
+    for (int j = 0; j < k; ++j) {
+      const int slot = pair_slot[t * k + j];
+      const float wj = w[t * k + j];
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(slot >= 0 ? y + (int64_t)slot * d + c : h + t * d + c);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) s[q] += wj * __uint_as_float((v[q >> 1] >> (16 * (q & 1))) << 16);
+    }
+    u32x4_t o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const __bf16 a = (__bf16)s[2 * q], b = (__bf16)s[2 * q + 1];
+      o[q] = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+    }
+    *reinterpret_cast<u32x4_t*>(out + t * d + c) = o;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -555,6 +580,9 @@ void sm_moe_combine(const void* y, const int* pair_slot, const float* w, int k, 
   if (f32)
     hipLaunchKernelGGL((moe_combine_kernel<float>), dim3(T), dim3(256), 0, stream, (const float*)y, pair_slot, w, k, d,
                        (float*)out, (const float*)h);
+  else if (d % 8 == 0 && (((uintptr_t)y | (uintptr_t)out | (uintptr_t)h) & 15) == 0)
+    hipLaunchKernelGGL(moe_combine_vec_kernel, dim3(T), dim3(256), 0, stream, (const bf16_t*)y, pair_slot, w, k, d,
+                       (bf16_t*)out, (const bf16_t*)h);
   else
     hipLaunchKernelGGL((moe_combine_kernel<bf16_t>), dim3(T), dim3(256), 0, stream, (const bf16_t*)y, pair_slot, w, k,
                        d, (bf16_t*)out, (const bf16_t*)h);

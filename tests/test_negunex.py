@@ -279,7 +279,21 @@ def _seq_meta(device, tables, q_lens, lens):
         tab[i, :len(t)] = t
     ti = lambda v: torch.tensor(v, dtype=torch.int32, device=device)  # noqa: E731
     return SeqMeta(n, ti(start), ti([0] * n), ti([0] * n), ti(row_seq), ti(row_len), tab.to(device),
-                   max_len=max(lens), max_q=max(q_lens), q_lens=list(q_lens))
+                   max_len=max(lens), max_q=max(q_lens), q_lens=list(q_lens), ctx_lens=list(lens))
+
+
+def test_attention_items_cover_every_token_once():
+    """The balanced order is a permutation of the plain cut; its blocks alternate direction."""
+    seq = _seq_meta("cpu", [torch.arange(20), torch.arange(3)], [1000, 130], [1200, 130])
+    plain = seq.attention_items(16).tolist()
+    snake = seq.attention_items(16, balance=8).tolist()
+    assert sorted(plain) == sorted(snake) and len(plain) == 63 + 9
+    assert sum(c for _, _, c in snake) == 1130
+    keys = [(1200 - 1000 if s == 0 else 0) + (t0 - (0 if s == 0 else 1000)) + c for s, t0, c in snake]
+    for b in range(0, len(keys), 8):
+        blk = keys[b:b + 8]
+        assert blk == sorted(blk, reverse=(b // 8) % 2 == 0)
+    assert max(keys[:8]) == 1200
 
 
 def _attention_oracle(q, rows, dim, row_len, scale, gate):
@@ -334,6 +348,18 @@ def test_one_key_stands_out(device, dtype, where, decode):
                                              (4, 2, 256, 256), (70, 1, 8, 8)])
 @pytest.mark.parametrize("decode_only", [False, True], ids=["mixed-step", "decode-step"])
 def test_grouped_attention_steps(device, dtype, Hq, Hkv, dim, vdim, decode_only):
+    _attention_steps(device, dtype, Hq, Hkv, dim, vdim, decode_only)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("Hq,Hkv,dim,vdim", [(6, 3, 24, 40), (8, 1, 64, 128), (5, 5, 10, 14), (4, 2, 256, 256)])
+def test_grouped_attention_128_row_items(Hq, Hkv, dim, vdim, monkeypatch):
+    """The optional form of the bf16 kernel with two blocks of 16 rows per wave."""
+    monkeypatch.setattr(sm, "GQA_RB2", True)
+    _attention_steps("cuda", torch.bfloat16, Hq, Hkv, dim, vdim, False)
+
+
+def _attention_steps(device, dtype, Hq, Hkv, dim, vdim, decode_only):
     """Several sequences of unequal length in one step, pages shuffled: single decoded tokens (one far
     beyond 256 keys, which cuts the keys into ranges on the matrix cores) beside prompt portions that
     start at 0, in mid-page and at a page border."""
