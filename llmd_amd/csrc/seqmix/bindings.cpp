@@ -304,14 +304,14 @@ void hyper_embed(Tensor ids, Tensor table, Tensor X) {
   TORCH_CHECK(table.is_cuda() && act_ok(table) && table.dim() == 2 && table.is_contiguous(), "table");
   CHECK_F32(X);
   const int T = ids.numel(), d = table.size(1);
-  TORCH_CHECK(X.dim() == 3 && X.size(0) >= 1 && X.size(0) <= 8 && X.size(1) == T && X.size(2) == d, "X [S <= 8, T, d]");
+  TORCH_CHECK(X.dim() == 3 && X.size(0) >= 1 && X.size(0) <= 16 && X.size(1) == T && X.size(2) == d, "X [S <= 16, T, d]");
   sm_hyper_embed(ids.data_ptr<int64_t>(), table.data_ptr(), table.size(0), X.data_ptr<float>(), X.size(0), T, d,
                  is_f32(table), cur());
 }
 
 void check_streams(const Tensor& X) {
   CHECK_F32(X);
-  TORCH_CHECK(X.dim() == 3 && X.size(0) >= 1 && X.size(0) <= 8 && X.size(2) <= 16384, "X [S <= 8, T, d <= 16384]");
+  TORCH_CHECK(X.dim() == 3 && X.size(0) >= 1 && X.size(0) <= 16 && X.size(2) <= 16384, "X [S <= 16, T, d <= 16384]");
 }
 
 void hyper_norm(Tensor X, Tensor w_in, Tensor norm_w, double eps, Tensor out) {

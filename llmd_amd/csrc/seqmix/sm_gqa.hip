@@ -309,8 +309,18 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   // row, value columns with lanes along the keys - both contiguous in the page. Keys at or beyond
   // kend are zeroed (a page's unwritten rest may hold anything, and 0 x NaN would spoil a column).
   u32x4_t pk[NCK], pv[NCV];
+  // one-page tiles: the tile's page and its first row in the page advance without a division
+  int tile_page = one_page ? kbeg / bs : 0, tile_off = one_page ? kbeg % bs : 0;
   auto fetch = [&](int k0) {
-    const int64_t page0 = one_page ? ((int64_t)bt[k0 / bs] * Hkv + g) * bs * Dr : 0;
+    const int64_t page0 = one_page ? ((int64_t)bt[tile_page] * Hkv + g) * bs * Dr : 0;
+    const int off0 = tile_off;
+    if (one_page) {
+      tile_off += MKT;
+      if (tile_off >= bs) {
+        tile_off = 0;
+        ++tile_page;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NCK; ++i) {
       const int e = threadIdx.x + i * NT;
@@ -319,7 +329,8 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       u32x4_t v = {0, 0, 0, 0};
       if (e < MKT * CK && c * 8 < dim && key < kend) {
         const int64_t page = one_page ? page0 : ((int64_t)bt[key / bs] * Hkv + g) * bs * Dr;
-        const bf16_t* src = cache + page + (int64_t)(key % bs) * dim + c * 8;
+        const int off = one_page ? off0 + j : key % bs;
+        const bf16_t* src = cache + page + (int64_t)off * dim + c * 8;
         if (vec) {
           v = *reinterpret_cast<const u32x4_t*>(src);
         } else {
@@ -338,7 +349,8 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       u32x4_t v = {0, 0, 0, 0};
       if (d < vdim && key < kend) {
         const int64_t page = one_page ? page0 : ((int64_t)bt[key / bs] * Hkv + g) * bs * Dr;
-        v = *reinterpret_cast<const u32x4_t*>(cache + page + (int64_t)bs * dim + (int64_t)d * bs + (key % bs));
+        const int off = one_page ? off0 + j8 * 8 : key % bs;
+        v = *reinterpret_cast<const u32x4_t*>(cache + page + (int64_t)bs * dim + (int64_t)d * bs + off);
         const int nv = kend - key;  // keys of this chunk that exist
         if (nv < 8) {
 #pragma unroll
@@ -403,22 +415,20 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       float psum = 0.f;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
-        // this lane's four weights are four consecutive keys: one 8-byte LDS write each for hi and lo
+        // this lane's four weights are four consecutive keys: one 8-byte LDS write each for hi and lo.
+        // hi = the weight's upper 16 bits (truncated), lo = the upper 16 bits of the exact rest:
+        // hi + lo differs from the fp32 weight by less than 2^-16 of it, with no rounding arithmetic.
         uint32_t hw[2], lw[2];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float pv = __builtin_amdgcn_exp2f(sc[rb][kb][r] - mref);
-          psum += pv;
-          const __bf16 hi = (__bf16)pv;
-          const __bf16 lo = (__bf16)(pv - (float)hi);
-          const uint32_t hb = __builtin_bit_cast(bf16_t, hi), lb = __builtin_bit_cast(bf16_t, lo);
-          if (r & 1) {
-            hw[r >> 1] |= hb << 16;
-            lw[r >> 1] |= lb << 16;
-          } else {
-            hw[r >> 1] = hb;
-            lw[r >> 1] = lb;
-          }
+        for (int r = 0; r < 4; r += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(sc[rb][kb][r] - mref);
+          const float p1 = __builtin_amdgcn_exp2f(sc[rb][kb][r + 1] - mref);
+          psum += p0 + p1;
+          const uint32_t u0 = __float_as_uint(p0), u1 = __float_as_uint(p1);
+          const uint32_t h0 = u0 & 0xffff0000u, h1 = u1 & 0xffff0000u;
+          const uint32_t r0 = __float_as_uint(p0 - __uint_as_float(h0)), r1 = __float_as_uint(p1 - __uint_as_float(h1));
+          hw[r >> 1] = (h0 >> 16) | h1;
+          lw[r >> 1] = (r0 >> 16) | (r1 & 0xffff0000u);
         }
         *reinterpret_cast<uint2*>(&ph[r16 * PS + kb * 16 + kq * 4]) = make_uint2(hw[0], hw[1]);
         *reinterpret_cast<uint2*>(&pl[r16 * PS + kb * 16 + kq * 4]) = make_uint2(lw[0], lw[1]);

@@ -18,7 +18,7 @@ using namespace sm;
 namespace {
 
 constexpr int NT = 256;
-constexpr int MAXS = 8;  // streams
+constexpr int MAXS = 16;  // streams
 
 template <typename T>
 __global__ __launch_bounds__(NT) void hyper_embed_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table,
