@@ -106,6 +106,96 @@ __global__ __launch_bounds__(NT) void hyper_update_norm_kernel(float* __restrict
   ln_row<T>(u, d, next_w, eps, out + t * d, red);
 }
 
+// Four columns per thread and step (d % 4 == 0, 16-byte aligned rows): the streams move as float4.
+__device__ __forceinline__ void ld4(const float* p, float (&v)[4]) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void ld4(const bf16_t* p, float (&v)[4]) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+__device__ __forceinline__ void st4(float* p, const float (&v)[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void st4(bf16_t* p, const float (&v)[4]) {
+  uint32_t w[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const __bf16 a = (__bf16)v[2 * i], b = (__bf16)v[2 * i + 1];  // round to nearest even
+    w[i] = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+  }
+  *reinterpret_cast<uint2*>(p) = make_uint2(w[0], w[1]);
+}
+
+constexpr int VMAXS = 4;  // streams of the float4 form
+
+template <typename T>
+__global__ __launch_bounds__(NT) void hyper_update_norm_vec_kernel(float* __restrict__ X, const T* __restrict__ y,
+                                                                   int64_t y_stride, const float* __restrict__ mix,
+                                                                   const float* __restrict__ w_out,
+                                                                   const float* __restrict__ next_in,
+                                                                   const T* __restrict__ next_w, float eps,
+                                                                   T* __restrict__ out, int S, int Tn, int d) {
+  extern __shared__ __attribute__((aligned(16))) float u[];
+  __shared__ float red[NT / 64];
+  __shared__ float sm_mix[VMAXS * VMAXS], sm_out[VMAXS], sm_in[VMAXS];
+  if (threadIdx.x < S * S) sm_mix[threadIdx.x] = mix[threadIdx.x];
+  if (threadIdx.x < S) {
+    sm_out[threadIdx.x] = w_out[threadIdx.x];
+    sm_in[threadIdx.x] = next_in ? next_in[threadIdx.x] : 0.f;
+  }
+  __syncthreads();
+  const int64_t t = blockIdx.x;
+  float psum = 0.f;
+  for (int c = threadIdx.x * 4; c < d; c += NT * 4) {
+    float x[VMAXS][4], yv[4], a[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < VMAXS; ++s)
+      if (s < S) ld4(X + ((int64_t)s * Tn + t) * d + c, x[s]);
+    ld4(y + t * y_stride + c, yv);
+#pragma unroll
+    for (int j = 0; j < VMAXS; ++j) {
+      if (j >= S) break;
+      float n[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = 0.f;
+#pragma unroll
+        for (int s = 0; s < VMAXS; ++s)
+          if (s < S) v += sm_mix[s * S + j] * x[s][i];   // the order of the scalar kernel
+        v += sm_out[j] * yv[i];
+        n[i] = v;
+        a[i] += sm_in[j] * v;
+      }
+      st4(X + ((int64_t)j * Tn + t) * d + c, n);
+    }
+    st4(u + c, a);
+    psum += (a[0] + a[1]) + (a[2] + a[3]);
+  }
+  if (next_w == nullptr) return;
+  // two-pass layer norm; a thread re-reads only the columns it wrote itself
+  const float mean = block_sum<NT>(psum, red) / (float)d;
+  float q = 0.f;
+  for (int c = threadIdx.x * 4; c < d; c += NT * 4) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float dv = u[c + i] - mean;
+      q += dv * dv;
+    }
+  }
+  const float var = block_sum<NT>(q, red) / (float)d;
+  const float inv = 1.f / sqrtf(var + eps);
+  for (int c = threadIdx.x * 4; c < d; c += NT * 4) {
+    float w[4], o[4];
+    ld4(next_w + c, w);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = (u[c + i] - mean) * inv * w[i];
+    st4(out + t * d + c, o);
+  }
+}
+
 template <typename T, int KIND>
 __global__ __launch_bounds__(NT) void gated_act_kernel(const T* __restrict__ gu, int64_t stride, int F,
                                                        T* __restrict__ out, int64_t n) {
@@ -152,6 +242,17 @@ void sm_hyper_update_norm(float* X, const void* y, int64_t y_stride, const float
                           hipStream_t stream) {
   if (T == 0) return;
   const size_t lds = (size_t)d * sizeof(float);
+  const size_t es = f32 ? 4 : 2;
+  if (S <= VMAXS && d % 4 == 0 && y_stride % 4 == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)y & (4 * es - 1)) == 0 &&
+      ((uintptr_t)next_w & (4 * es - 1)) == 0 && ((uintptr_t)out & (4 * es - 1)) == 0) {
+    if (f32)
+      hipLaunchKernelGGL((hyper_update_norm_vec_kernel<float>), dim3(T), dim3(NT), lds, stream, X, (const float*)y,
+                         y_stride, mix, w_out, next_in, (const float*)next_w, eps, (float*)out, S, T, d);
+    else
+      hipLaunchKernelGGL((hyper_update_norm_vec_kernel<bf16_t>), dim3(T), dim3(NT), lds, stream, X, (const bf16_t*)y,
+                         y_stride, mix, w_out, next_in, (const bf16_t*)next_w, eps, (bf16_t*)out, S, T, d);
+    return;
+  }
   if (f32)
     hipLaunchKernelGGL((hyper_update_norm_kernel<float>), dim3(T), dim3(NT), lds, stream, X, (const float*)y, y_stride,
                        mix, w_out, next_in, (const float*)next_w, eps, (float*)out, S, T, d);

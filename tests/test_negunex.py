@@ -155,7 +155,7 @@ def _pages_of(rows, dim):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("S,d", [(1, 40), (2, 33), (5, 300), (11, 24)])
+@pytest.mark.parametrize("S,d", [(1, 40), (2, 33), (5, 300), (11, 24), (3, 64), (4, 2052)])
 def test_streams_and_layer_norm(device, S, d):
     g = torch.Generator().manual_seed(S)
     T = 7
