@@ -21,6 +21,7 @@
 // Both forms multiply the result by sigmoid(gate) when a gate is given. A row's result depends
 // only on its own keys and the fixed tile sizes.
 #include "seqmix_common.h"
+#include <algorithm>
 
 using namespace sm;
 
@@ -43,7 +44,9 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
   const int64_t slot = slots[t];
   const int Dr = dim + vdim;
   const int64_t blk = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
-  for (int hd = wave; hd < Hq + Hkv; hd += NT / 64) {
+  // blockIdx.y spreads a token's heads (a wave each) and value elements over workgroups: a step of
+  // few tokens still fills the chip
+  for (int hd = blockIdx.y * (NT / 64) + wave; hd < Hq + Hkv; hd += gridDim.y * (NT / 64)) {
     const bool is_q = hd < Hq;
     const int col0 = is_q ? hd * dim : Hq * dim + (hd - Hq) * dim;
     float r[MAXE];
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
     }
   }
   const int nv = Hkv * vdim, vcol0 = (Hq + Hkv) * dim;
-  for (int e = threadIdx.x; e < nv; e += NT) {
+  for (int e = blockIdx.y * NT + threadIdx.x; e < nv; e += gridDim.y * NT) {
     float v = ld(row + vcol0 + e) + (bias ? bias[vcol0 + e] : 0.f);
     if (v_mode == 1) v_first[t * nv + e] = v;
     else if (v_mode == 2) v = (1.f - lam) * v + lam * v_first[t * nv + e];
@@ -568,12 +571,16 @@ void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const
                        int unit, float eps, float* v_first, int v_mode, float lam, const int64_t* slots, void* cache,
                        int bs, void* q_out, int T, int f32, hipStream_t stream) {
   if (T == 0) return;
+  // workgroups per token: all heads in parallel for small steps, fewer as the step grows
+  const int per_tok = (Hq + Hkv + NT / 64 - 1) / (NT / 64);
+  const int gy = std::max(1, std::min(per_tok, 4096 / T));
+  const dim3 grid(T, gy);
   if (f32)
-    hipLaunchKernelGGL((qkv_rope_cache_kernel<float>), dim3(T), dim3(NT), 0, stream, (const float*)qkv, stride, bias,
+    hipLaunchKernelGGL((qkv_rope_cache_kernel<float>), grid, dim3(NT), 0, stream, (const float*)qkv, stride, bias,
                        positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
                        slots, (float*)cache, bs, (float*)q_out);
   else
-    hipLaunchKernelGGL((qkv_rope_cache_kernel<bf16_t>), dim3(T), dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias,
+    hipLaunchKernelGGL((qkv_rope_cache_kernel<bf16_t>), grid, dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias,
                        positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
                        slots, (bf16_t*)cache, bs, (bf16_t*)q_out);
 }

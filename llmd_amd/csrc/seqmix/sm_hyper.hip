@@ -210,6 +210,31 @@ __global__ __launch_bounds__(NT) void gated_act_kernel(const T* __restrict__ gu,
   st(out + i, a * v);
 }
 
+// bf16, F % 8 == 0, 16-byte aligned rows: eight columns per thread from 16-byte loads.
+template <int KIND>
+__global__ __launch_bounds__(NT) void gated_act_vec_kernel(const bf16_t* __restrict__ gu, int64_t stride, int F,
+                                                           bf16_t* __restrict__ out, int64_t n8) {
+  const int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x;
+  if (i >= n8) return;
+  const int f8 = F / 8;
+  const int64_t t = i / f8;
+  const int j = (int)(i - t * f8) * 8;
+  float g[8], v[8], o[8];
+  ld4(gu + t * stride + j, *reinterpret_cast<float(*)[4]>(&g[0]));
+  ld4(gu + t * stride + j + 4, *reinterpret_cast<float(*)[4]>(&g[4]));
+  ld4(gu + t * stride + F + j, *reinterpret_cast<float(*)[4]>(&v[0]));
+  ld4(gu + t * stride + F + j + 4, *reinterpret_cast<float(*)[4]>(&v[4]));
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    float a;
+    if (KIND == 0) a = 0.5f * g[q] * (1.f + tanhf(0.7978845608028654f * (g[q] + 0.044715f * g[q] * g[q] * g[q])));
+    else a = g[q] / (1.f + expf(-g[q]));
+    o[q] = a * v[q];
+  }
+  st4(out + t * F + j, *reinterpret_cast<float(*)[4]>(&o[0]));
+  st4(out + t * F + j + 4, *reinterpret_cast<float(*)[4]>(&o[4]));
+}
+
 }  // namespace
 
 extern "C" {
@@ -264,6 +289,15 @@ void sm_hyper_update_norm(float* X, const void* y, int64_t y_stride, const float
 void sm_gated_act(const void* gu, int64_t stride, int F, int kind, void* out, int T, int f32, hipStream_t stream) {
   const int64_t n = (int64_t)T * F;
   if (n == 0) return;
+  if (!f32 && F % 8 == 0 && stride % 8 == 0 && (((uintptr_t)gu | (uintptr_t)out) & 15) == 0) {
+    const int64_t n8 = n / 8;
+    const dim3 g8((unsigned)((n8 + NT - 1) / NT));
+    if (kind == 0)
+      hipLaunchKernelGGL((gated_act_vec_kernel<0>), g8, dim3(NT), 0, stream, (const bf16_t*)gu, stride, F, (bf16_t*)out, n8);
+    else
+      hipLaunchKernelGGL((gated_act_vec_kernel<1>), g8, dim3(NT), 0, stream, (const bf16_t*)gu, stride, F, (bf16_t*)out, n8);
+    return;
+  }
   const dim3 grid((unsigned)((n + NT - 1) / NT));
 #define SM_GO(TYPE, K) \
   hipLaunchKernelGGL((gated_act_kernel<TYPE, K>), grid, dim3(NT), 0, stream, (const TYPE*)gu, stride, F, (TYPE*)out, n)

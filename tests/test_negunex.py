@@ -445,6 +445,10 @@ def test_gated_activation(device, kind):
     got = sm.gated_act(_dev(gu, device), 37, kind)
     act = oracle.gelu_tanh if kind == "gelu_tanh" else oracle.silu
     assert rel_err(got, act(gu[:, :37].double()) * gu[:, 37:74].double()) < 1e-5
+    # bfloat16 rows of 16-byte multiples (the vector form on the GPU)
+    gb = (torch.randn(9, 2 * 48, generator=g) * 3).to(torch.bfloat16)
+    got = sm.gated_act(_dev(gb, device), 48, kind)
+    assert rel_err(got.float(), act(gb[:, :48].double()) * gb[:, 48:].double()) < 1e-2
 
 
 # ------------------------------------------------------------------ the model on the engine
