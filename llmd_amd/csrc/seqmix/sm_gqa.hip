@@ -248,8 +248,12 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int DkP = 32 * NKS, VP = 16 * NCB;
   constexpr int KS = DkP + 8, VS = MKT + 8, PS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
-  __shared__ __attribute__((aligned(16))) bf16_t sK[MKT * KS];
-  __shared__ __attribute__((aligned(16))) bf16_t sVt[VP * VS];
+  // Two tile buffers for the small forms: the next tile is written while the current one is read and
+  // one barrier per tile is enough. The 256 / 256 form keeps one buffer (two would leave one
+  // workgroup per CU) and brackets the write with two barriers.
+  constexpr int NBUF = NKS <= 4 ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) bf16_t sK[NBUF * MKT * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t sVt[NBUF * VP * VS];
   __shared__ __attribute__((aligned(16))) bf16_t sP[2 * RB * 4 * 16 * PS];  // [hi | lo][rb][wave][16][PS]
   // the kv head is the fastest grid index: the workgroups of one item follow each other
   const int item = blockIdx.y, g = blockIdx.x, G = Hq / Hkv, Dr = dim + vdim;
@@ -269,8 +273,8 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   const int maxlen = row_len[tok0 + ntok - 1];  // the run's last token sees the most keys
 
   // padding columns of the key tile and padding rows of the value tile stay zero for the whole kernel
-  for (int e = threadIdx.x; e < MKT * KS; e += NT) sK[e] = 0;
-  for (int e = threadIdx.x; e < VP * VS; e += NT) sVt[e] = 0;
+  for (int e = threadIdx.x; e < NBUF * MKT * KS; e += NT) sK[e] = 0;
+  for (int e = threadIdx.x; e < NBUF * VP * VS; e += NT) sVt[e] = 0;
 
   bf16x8_t qf[RB][NKS];
 #pragma unroll
@@ -363,23 +367,40 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       pv[i] = v;
     }
   };
-  if (kbeg < kend) fetch(kbeg);
-  for (int k0 = kbeg; k0 < kend; k0 += MKT) {
-    __syncthreads();  // the previous tile is no longer read (first time: the zero fill is done)
+  auto stage = [&](int buf) {  // the fetched tile -> LDS buffer buf
+    bf16_t* const kb_ = sK + buf * MKT * KS;
+    bf16_t* const vb_ = sVt + buf * VP * VS;
 #pragma unroll
     for (int i = 0; i < NCK; ++i) {
       const int e = threadIdx.x + i * NT;
       const int j = e / CK, c = e - j * CK;
-      if (e < MKT * CK && c * 8 < dim) *reinterpret_cast<u32x4_t*>(&sK[j * KS + c * 8]) = pk[i];
+      if (e < MKT * CK && c * 8 < dim) *reinterpret_cast<u32x4_t*>(&kb_[j * KS + c * 8]) = pk[i];
     }
 #pragma unroll
     for (int i = 0; i < NCV; ++i) {
       const int e = threadIdx.x + i * NT;
       const int d = e / CV, j8 = e - d * CV;
-      if (d < vdim) *reinterpret_cast<u32x4_t*>(&sVt[d * VS + j8 * 8]) = pv[i];
+      if (d < vdim) *reinterpret_cast<u32x4_t*>(&vb_[d * VS + j8 * 8]) = pv[i];
     }
+  };
+  if (kbeg < kend) fetch(kbeg);
+  if (NBUF == 2) {
+    __syncthreads();  // the zero fill is done
+    stage(0);
+    if (kbeg + MKT < kend) fetch(kbeg + MKT);
     __syncthreads();
-    if (k0 + MKT < kend) fetch(k0 + MKT);  // in flight during this tile's products
+  }
+  int it = 0;
+  for (int k0 = kbeg; k0 < kend; k0 += MKT, ++it) {
+    const int cur = NBUF == 2 ? (it & 1) : 0;
+    if (NBUF == 1) {
+      __syncthreads();  // the previous tile is no longer read (first time: the zero fill is done)
+      stage(0);
+      __syncthreads();
+      if (k0 + MKT < kend) fetch(k0 + MKT);  // in flight during this tile's products
+    }
+    const bf16_t* const tK = sK + cur * MKT * KS;
+    const bf16_t* const tV = sVt + cur * VP * VS;
     // scores of this lane's rows against keys k0 + 16 kb + 4 kq + r
     float sc[RB][2][4];
 #pragma unroll
@@ -389,7 +410,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       for (int rb = 0; rb < RB; ++rb) a[rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
-        const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(&sK[(kb * 16 + r16) * KS + ks * 32 + kq * 8]);
+        const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(&tK[(kb * 16 + r16) * KS + ks * 32 + kq * 8]);
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) a[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[rb][ks], a[rb], 0, 0, 0);
       }
@@ -456,7 +477,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     }
 #pragma unroll
     for (int n = 0; n < NCB; ++n) {
-      const bf16x8_t vb = *reinterpret_cast<const bf16x8_t*>(&sVt[(n * 16 + r16) * VS + kq * 8]);
+      const bf16x8_t vb = *reinterpret_cast<const bf16x8_t*>(&tV[(n * 16 + r16) * VS + kq * 8]);
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         f32x4_t acc = o[rb][n];
@@ -468,6 +489,15 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pal[rb], vb, acc, 0, 0, 0);
         o[rb][n] = acc;
       }
+    }
+    if (NBUF == 2) {
+      // every wave has finished the previous tile (barrier below, one iteration ago), so the other
+      // buffer is free: write the next tile there and ask for the one after it
+      if (k0 + MKT < kend) {
+        stage(cur ^ 1);
+        if (k0 + 2 * MKT < kend) fetch(k0 + 2 * MKT);
+      }
+      __syncthreads();
     }
   }
   // o[rb][n][r] = O[row 16 (4 rb + wave) + 4 kq + r][column 16 n + r16]
