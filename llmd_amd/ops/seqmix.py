@@ -252,6 +252,7 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
 
 
 GQA_MFMA = os.environ.get("LLMD_GQA_MFMA", "1") == "1"
+GQA_DECODE_WGS = int(os.environ.get("LLMD_GQA_DECODE_WGS", "2048"))  # workgroups a decode-only step aims for
 # LLMD_GQA_RB2=1: prompt portions run as 128-row items, two blocks of 16 rows per wave. Measured slower
 # than 64-row items at 128/128 heads (2048-token prompt: 227 us against 181 us - 185 + 64 registers
 # leave two waves per SIMD instead of three), so it stays an option.
@@ -281,7 +282,7 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
             # decode-only step: key ranges so that items x kv heads x ranges give the chip about
             # eight workgroups per CU (a workgroup walks its tiles one after another)
             n = items.shape[0] * Hkv
-            nsplit = max(1, min(-(-2048 // n), seq.max_len // 128))
+            nsplit = max(1, min(-(-GQA_DECODE_WGS // n), seq.max_len // 128))
             split = -(-seq.max_len // (nsplit * 32)) * 32
             nsplit = -(-seq.max_len // split)
             if nsplit > 1:
