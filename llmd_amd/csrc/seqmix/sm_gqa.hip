@@ -16,7 +16,7 @@
 //   the group) rows of one sequence and kv head, one or two blocks of 16 rows per wave. Key tiles of
 //   32 in LDS (keys row-major, values transposed as in the cache), S^T = K Q^T and O += P V on
 //   v_mfma_f32_16x16x32_bf16; fp32 online softmax in base 2; P enters the second product as a bf16
-//   pair (hi + lo). Decode-only steps cut the keys into ranges over blockIdx.z and a merge kernel
+//   pair (hi + lo) straight from the registers the scores arrive in. Decode-only steps cut the keys into ranges over blockIdx.z and a merge kernel
 //   joins them.
 // Both forms multiply the result by sigmoid(gate) when a gate is given. A row's result depends
 // only on its own keys and the fixed tile sizes.
@@ -247,14 +247,13 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     const bf16_t* __restrict__ gate, int64_t gate_stride, bf16_t* __restrict__ out, int split_keys,
     float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int DkP = 32 * NKS, VP = 16 * NCB;
-  constexpr int KS = DkP + 8, VS = MKT + 8, PS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
+  constexpr int KS = DkP + 8, VS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
   // Two tile buffers for the small forms: the next tile is written while the current one is read and
   // one barrier per tile is enough. The 256 / 256 form keeps one buffer (two would leave one
   // workgroup per CU) and brackets the write with two barriers.
   constexpr int NBUF = NKS <= 4 ? 2 : 1;
   __shared__ __attribute__((aligned(16))) bf16_t sK[NBUF * MKT * KS];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[NBUF * VP * VS];
-  __shared__ __attribute__((aligned(16))) bf16_t sP[2 * RB * 4 * 16 * PS];  // [hi | lo][rb][wave][16][PS]
   // the kv head is the fastest grid index: the workgroups of one item follow each other
   const int item = blockIdx.y, g = blockIdx.x, G = Hq / Hkv, Dr = dim + vdim;
   const int seq = items[item * 3], tok0 = items[item * 3 + 1], ntok = items[item * 3 + 2];
@@ -380,7 +379,13 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     for (int i = 0; i < NCV; ++i) {
       const int e = threadIdx.x + i * NT;
       const int d = e / CV, j8 = e - d * CV;
-      if (d < vdim) *reinterpret_cast<u32x4_t*>(&vb_[d * VS + j8 * 8]) = pv[i];
+      // a value column's keys are stored in the order the weights arrive in: position 8 q + i holds
+      // key 4 q + i (i < 4) or key 16 + 4 q + i - 4, so one 16-byte read gives a lane its eight keys
+      if (d < vdim) {
+        const int base = d * VS + (j8 & 1) * 16 + (j8 >> 1) * 4;
+        *reinterpret_cast<uint2*>(&vb_[base]) = make_uint2(pv[i][0], pv[i][1]);
+        *reinterpret_cast<uint2*>(&vb_[base + 8]) = make_uint2(pv[i][2], pv[i][3]);
+      }
     }
   };
   if (kbeg < kend) fetch(kbeg);
@@ -420,12 +425,16 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
         for (int r = 0; r < 4; ++r)
           sc[rb][kb][r] = (k0 + kb * 16 + kq * 4 + r < min(mylen[rb], kend)) ? a[rb][r] * scale2 : -INFINITY;
     }
+    // The weights never pass through LDS. After S^T = K Q^T this lane holds, for its query row r16,
+    // the keys 4 kq .. 4 kq + 3 of both 16-key halves of the tile - eight keys, which is exactly one
+    // A operand of the second product if the contraction index is ordered that way; the value
+    // operand below is read in the same order (the order of a contraction is free as long as both
+    // operands agree).
     float cr[RB][4];
     bool rescale[RB];  // wave-uniform: some row's maximum moved in this tile
+    bf16x8_t pah[RB], pal[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      bf16_t* ph = sP + ((rb * 4 + wave) * 16) * PS;
-      bf16_t* pl = ph + RB * 4 * 16 * PS;
       float mx = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
@@ -437,12 +446,11 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       const float mref = (mn == -INFINITY) ? 0.f : mn;  // a row with no key yet
       const float corr = __builtin_amdgcn_exp2f(m[rb] - mref);
       float psum = 0.f;
+      u32x4_t hw, lw;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
-        // this lane's four weights are four consecutive keys: one 8-byte LDS write each for hi and lo.
         // hi = the weight's upper 16 bits (truncated), lo = the upper 16 bits of the exact rest:
         // hi + lo differs from the fp32 weight by less than 2^-16 of it, with no rounding arithmetic.
-        uint32_t hw[2], lw[2];
 #pragma unroll
         for (int r = 0; r < 4; r += 2) {
           const float p0 = __builtin_amdgcn_exp2f(sc[rb][kb][r] - mref);
@@ -451,12 +459,12 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
           const uint32_t u0 = __float_as_uint(p0), u1 = __float_as_uint(p1);
           const uint32_t h0 = u0 & 0xffff0000u, h1 = u1 & 0xffff0000u;
           const uint32_t r0 = __float_as_uint(p0 - __uint_as_float(h0)), r1 = __float_as_uint(p1 - __uint_as_float(h1));
-          hw[r >> 1] = (h0 >> 16) | h1;
-          lw[r >> 1] = (r0 >> 16) | (r1 & 0xffff0000u);
+          hw[kb * 2 + (r >> 1)] = (h0 >> 16) | h1;
+          lw[kb * 2 + (r >> 1)] = (r0 >> 16) | (r1 & 0xffff0000u);
         }
-        *reinterpret_cast<uint2*>(&ph[r16 * PS + kb * 16 + kq * 4]) = make_uint2(hw[0], hw[1]);
-        *reinterpret_cast<uint2*>(&pl[r16 * PS + kb * 16 + kq * 4]) = make_uint2(lw[0], lw[1]);
       }
+      pah[rb] = __builtin_bit_cast(bf16x8_t, hw);
+      pal[rb] = __builtin_bit_cast(bf16x8_t, lw);
       psum += __shfl_xor(psum, 16, 64);
       psum += __shfl_xor(psum, 32, 64);
       l[rb] = l[rb] * corr + psum;
@@ -465,15 +473,6 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) cr[rb][r] = __shfl(corr, kq * 4 + r, 64);
       rescale[rb] = __any(corr != 1.f);
-    }
-    // P is written and read by the same wave only: LDS operations of a wave complete in order
-    __builtin_amdgcn_wave_barrier();
-    bf16x8_t pah[RB], pal[RB];
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const bf16_t* ph = sP + ((rb * 4 + wave) * 16) * PS;
-      pah[rb] = *reinterpret_cast<const bf16x8_t*>(&ph[r16 * PS + kq * 8]);
-      pal[rb] = *reinterpret_cast<const bf16x8_t*>(&ph[RB * 4 * 16 * PS + r16 * PS + kq * 8]);
     }
 #pragma unroll
     for (int n = 0; n < NCB; ++n) {
