@@ -102,6 +102,105 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
   }
 }
 
+// bf16 form with 16-byte accesses: a head is dim / 8 lanes, each with eight consecutive elements (four
+// interleaved pairs, or one eighth of a half with its partner chunk loaded beside it). Needs
+// dim = 8 * 2^k <= 512, rotary dims a multiple of 8 (16 for the half-split pairing) and 16-byte
+// aligned rows; the launcher falls back to the element-wise kernel otherwise.
+__device__ __forceinline__ void ld8(const bf16_t* p, float (&v)[8]) {
+  const uint4 t = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ void add8(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w;
+  v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
+}
+__device__ __forceinline__ void st8(bf16_t* p, const float (&v)[8], float mul) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const __bf16 a = (__bf16)(v[2 * i] * mul), b = (__bf16)(v[2 * i + 1] * mul);  // round to nearest even
+    w[i] = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+  }
+  *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__global__ __launch_bounds__(NT) void qkv_rope_cache_vec_kernel(
+    const bf16_t* __restrict__ qkv, int64_t stride, const float* __restrict__ bias,
+    const int64_t* __restrict__ positions, const float* __restrict__ cos_sin, int Hq, int Hkv, int dim, int vdim,
+    int rot_dims, int interleaved, int unit, float eps, float* __restrict__ v_first, int v_mode, float lam,
+    const int64_t* __restrict__ slots, bf16_t* __restrict__ cache, int bs, bf16_t* __restrict__ q_out) {
+  const int64_t t = blockIdx.x;
+  const int half = rot_dims >> 1;
+  const float* cs = rot_dims ? cos_sin + positions[t] * rot_dims : nullptr;  // [cos(half) | sin(half)]
+  const bf16_t* row = qkv + t * stride;
+  const int64_t slot = slots[t];
+  const int Dr = dim + vdim;
+  const int64_t blk = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
+  const int lph = dim >> 3, hpp = NT / lph;  // lanes per head, heads per pass
+  const int c = threadIdx.x & (lph - 1), hl = threadIdx.x / lph;
+  for (int h0 = blockIdx.y * hpp; h0 < Hq + Hkv; h0 += gridDim.y * hpp) {
+    const int hd = h0 + hl;
+    const bool on = hd < Hq + Hkv;
+    const int col = hd * dim + c * 8;  // q heads, then k heads, back to back in the projection
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (on) {
+      ld8(row + col, x);
+      if (bias) add8(bias + col, x);
+      if (c * 8 < rot_dims) {
+        if (interleaved) {
+          const float4 co = *reinterpret_cast<const float4*>(cs + c * 4);
+          const float4 si = *reinterpret_cast<const float4*>(cs + half + c * 4);
+          const float cc[4] = {co.x, co.y, co.z, co.w}, sn[4] = {si.x, si.y, si.z, si.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float u = x[2 * i], v = x[2 * i + 1];
+            x[2 * i] = u * cc[i] - v * sn[i];
+            x[2 * i + 1] = v * cc[i] + u * sn[i];
+          }
+        } else {
+          const bool first = c * 8 < half;
+          const int pc = first ? col + half : col - half;  // the partner chunk
+          const int f = first ? c * 8 : c * 8 - half;
+          float xp[8], cc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, sn[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          ld8(row + pc, xp);
+          if (bias) add8(bias + pc, xp);
+          add8(cs + f, cc);
+          add8(cs + half + f, sn);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) x[i] = first ? x[i] * cc[i] - xp[i] * sn[i] : x[i] * cc[i] + xp[i] * sn[i];
+        }
+      }
+    }
+    float inv = 1.f;
+    if (unit) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+      for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);  // the head's lanes are an aligned group
+      inv = 1.f / sqrtf(ss / (float)dim + eps);
+    }
+    if (!on) continue;
+    if (hd < Hq) st8(q_out + (t * Hq + hd) * dim + c * 8, x, inv);
+    else if (slot >= 0) st8(cache + (blk * Hkv + (hd - Hq)) * bs * Dr + off * dim + c * 8, x, inv);
+  }
+  const int nv = Hkv * vdim, vcol0 = (Hq + Hkv) * dim;
+  for (int e = blockIdx.y * NT + threadIdx.x; e < nv; e += gridDim.y * NT) {
+    float v = ld(row + vcol0 + e) + (bias ? bias[vcol0 + e] : 0.f);
+    if (v_mode == 1) v_first[t * nv + e] = v;
+    else if (v_mode == 2) v = (1.f - lam) * v + lam * v_first[t * nv + e];
+    if (slot >= 0) {
+      const int g = e / vdim, cc = e - g * vdim;
+      st(cache + (blk * Hkv + g) * bs * Dr + (int64_t)bs * dim + (int64_t)cc * bs + off, v);  // transposed
+    }
+  }
+}
+
 // VC = ceil(vdim / 64) output columns per lane; QT token rows per workgroup.
 template <typename T, int VC, int QT>
 __global__ __launch_bounds__(NT) void grouped_attention_kernel(
@@ -608,7 +707,17 @@ void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const
     hipLaunchKernelGGL((qkv_rope_cache_kernel<float>), grid, dim3(NT), 0, stream, (const float*)qkv, stride, bias,
                        positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
                        slots, (float*)cache, bs, (float*)q_out);
-  else
+  else if (dim % 8 == 0 && dim <= 512 && ((dim >> 3) & ((dim >> 3) - 1)) == 0 && stride % 8 == 0 &&
+           rot_dims % (interleaved ? 8 : 16) == 0 &&
+           (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)cache | (uintptr_t)bias | (uintptr_t)cos_sin) & 15) == 0) {
+    // a pass covers 256 / (dim / 8) heads: fewer workgroups per token than the element-wise form
+    const int hpp = NT / (dim >> 3);
+    const int per_tok_v = (Hq + Hkv + hpp - 1) / hpp;
+    const dim3 vgrid(T, std::max(1, std::min(per_tok_v, 4096 / T)));
+    hipLaunchKernelGGL(qkv_rope_cache_vec_kernel, vgrid, dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias, positions,
+                       cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam, slots,
+                       (bf16_t*)cache, bs, (bf16_t*)q_out);
+  } else
     hipLaunchKernelGGL((qkv_rope_cache_kernel<bf16_t>), grid, dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias,
                        positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
                        slots, (bf16_t*)cache, bs, (bf16_t*)q_out);

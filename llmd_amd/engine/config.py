@@ -352,6 +352,21 @@ _register(ModelConfig(model_type="deepseek", name="tiny-deepseek", hidden_size=2
                       qk_rope_head_dim=64, v_head_dim=128, head_dim=192, bos_token_id=1, eos_token_id=2))
 
 
+def _tiny_negunex() -> ModelConfig:
+    att = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 32 ** -0.5, "v_mix": True,
+           "rot": {"dims": 16, "base": 10000.0, "scaling": {"factor": 2.0, "low": 1.0, "high": 4.0, "original": 256}}}
+    return negunex_config({
+        "architecture": "Negunex", "name": "tiny-negunex", "width": 128, "vocab": 512, "streams": 2,
+        "norm": {"eps": 1e-6}, "max_position": 4096, "eos": 1,
+        "layers": [{"type": "attention", "mixer": att, "mlp": {"kind": "dense", "ff": 256}},
+                   {"type": "attention", "mixer": att,
+                    "mlp": {"kind": "moe", "expert": {"ff": 64}, "router": {"experts": 6, "identity": 2, "top": 2}}},
+                   {"type": "attention", "mixer": dict(att, v_mix=False), "mlp": None}]})
+
+
+_register(_tiny_negunex())
+
+
 def get_model_config(name_or_path: str) -> ModelConfig:
     if name_or_path in PRESETS:
         return dataclasses.replace(PRESETS[name_or_path])
