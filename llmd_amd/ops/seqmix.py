@@ -1,6 +1,8 @@
 """Ops of per-layer ("sequence mixer") stacks: latent attention of any size, the selective
 scan, the generalized delta rule, zero-centred norms with layer scale, depth averaging, plain
-(ungated) expert feed-forwards.
+(ungated) expert feed-forwards; hyper-connected residual streams with layer norm, grouped-query
+attention with its own key and value sizes (bias, rotary, unit norm, value mixing, gate), gated
+activations, score routing with a selection-only correction, gated experts with identity experts.
 
 GPU tensors go to the ``llmd_amd._C_seqmix`` library (csrc/seqmix/*.hip, built on its own so a
 model that needs only these kernels compiles only these); it is templated on the activation
